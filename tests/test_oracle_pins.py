@@ -1,0 +1,291 @@
+"""Pins the CPU oracle (oracle/anchor_oracle.py) with checks that do not retype its formulas:
+float64 brute force over explicit key sets, a literal walk of the reference's two tile loops,
+library softmax attention, closed forms at theta -> +/-inf, torch's own bf16 cast."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from anchor_attn.synthetic import make_qkv
+from oracle import anchor_oracle as ao
+
+D = 128
+S = 2048
+SM = 1.0 / math.sqrt(D)
+
+
+def _np(*ts):
+    return [t.float().numpy() for t in ts]
+
+
+@pytest.fixture(scope="module")
+def small():
+    """N = 3 big blocks, GQA 2:1, 96 stripes: bb = 0, 1 and 2 are all exercised."""
+    q, k, v, pos = make_qkv(3 * S, 2, 1, n_stripes=96, seed=11)
+    Q, K, V = _np(q, k, v)
+    res = ao.anchor_attn_reference(Q, K, V, difference=12.0)
+    return Q, K, V, pos.numpy(), res
+
+
+# ---------------------------------------------------------------- bf16 rounding and scale chains
+def test_rn16_matches_torch_cast():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(200000, generator=g) * torch.logspace(-30, 30, 200000)
+    bits = torch.randint(0, 2**31 - 1, (200000,), generator=g, dtype=torch.int64).to(torch.int32)
+    y = bits.view(torch.float32)
+    ties = (torch.arange(1, 4097, dtype=torch.int32) << 16 | 0x8000).view(torch.float32)  # exact ties
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1e-40, -1e-40, 3.3895e38])
+    for t in (x, y[torch.isfinite(y)], ties, special):
+        want = t.to(torch.bfloat16).float().numpy()
+        got = ao.rn16(t.numpy())
+        assert np.array_equal(want.view(np.uint32), got.view(np.uint32))
+    assert np.isnan(ao.rn16(np.array([np.nan], np.float32))[0])
+
+
+def test_scale_chain_constants_and_torch_bf16_arithmetic():
+    # constants the stage-1 chain rounds to for D=128
+    assert float(ao.rn16(np.array([SM], np.float32))[0]) == 0.08837890625
+    assert float(ao.rn16(np.array([ao.LOG2E], np.float32))[0]) == 1.4453125
+    q = torch.randn(4096, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    # torch evaluates bf16*bf16 as a float32 product rounded once to bf16
+    t1 = (q * torch.tensor(SM, dtype=torch.bfloat16)) * torch.tensor(ao.LOG2E, dtype=torch.bfloat16)
+    assert t1.dtype == torch.bfloat16
+    assert np.array_equal(t1.float().numpy(), ao.q1_scale_chain(q.float().numpy(), SM))
+    t3 = ((q.float() * torch.tensor(SM, dtype=torch.float32)) * torch.tensor(ao.LOG2E, dtype=torch.float32)).to(torch.bfloat16)
+    assert np.array_equal(t3.float().numpy(), ao.q3_scale_chain(q.float().numpy(), SM))
+    # the two chains really differ (that is why both exist): ratio ~1.0017
+    r = ao.q1_scale_chain(np.full(1, 64.0, np.float32), SM)[0] / (64.0 * SM * ao.LOG2E)
+    assert abs(r - 1.0017) < 2e-3 and r != 1.0
+
+
+# ---------------------------------------------------------------- stage 1
+def _literal_stage1_block(Qh, Kh, Vh, m_idx, sm_scale, block=128, step=16):
+    """Walk the two loops of the reference's stage-1 program for ONE 128-query block exactly as
+    written (loop bounds, pointer start/advance, additive mask) in float64; returns (M, L, Acc).
+    anchor_step_1_2_v2.py:42-44 (offsets), :97-112 (local pointers), :125-156 (loops)."""
+    big = (m_idx * block) // (block * step)
+    init_offset = min(1 * block * step, (m_idx + 1) * block)
+    local_offset = max((big - 1 + 1) * block * step, 0)
+    rows = np.arange(m_idx * block, (m_idx + 1) * block)
+    q = ao.q1_scale_chain(Qh[rows], sm_scale).astype(np.float64)
+    m = np.full(block, -np.inf)
+    l = np.zeros(block)
+    acc = np.zeros((block, Qh.shape[1]))
+
+    def tile(kptr, j, m, l, acc):
+        s = q @ Kh[kptr : kptr + block].astype(np.float64).T
+        s = s + np.where((np.arange(block)[None, :] + j) <= rows[:, None], 0.0, -1e6)
+        m_new = np.maximum(m, s.max(1))
+        p = np.exp2(s - m_new[:, None])
+        a = np.exp2(m - m_new)
+        return m_new, l * a + p.sum(1), acc * a[:, None] + p @ Vh[kptr : kptr + block].astype(np.float64)
+
+    kptr = 0
+    for j in range(0, init_offset, block):
+        m, l, acc = tile(kptr, j, m, l, acc)
+        kptr += block
+    kptr = local_offset
+    for j in range(max(local_offset, init_offset), (big + 1) * block * step, block):
+        m, l, acc = tile(kptr, j, m, l, acc)
+        kptr += block
+    return m, l, acc
+
+
+def _window_mask(N):
+    """W(r) = [0,S) U [bb*S, r] for bb>=1, [0,r] for bb=0, built straight from that sentence."""
+    r = np.arange(N)[:, None]
+    j = np.arange(N)[None, :]
+    bb = r // S
+    return (j <= r) & ((j < S) | (j >= bb * S))
+
+
+def test_stage1_literal_walk_equals_window_closed_form(small):
+    Q, K, V, _, res = small
+    N = Q.shape[2]
+    mask = _window_mask(N)
+    for h in range(2):
+        q1 = ao.q1_scale_chain(Q[0, h], SM).astype(np.float64)
+        s = q1 @ K[0, 0].astype(np.float64).T
+        s[~mask] = -np.inf
+        M = s.max(1)
+        P = np.exp2(s - M[:, None])
+        L = P.sum(1)
+        A = P @ V[0, 0].astype(np.float64)
+        # (a) the literal loop walk gives the closed-form key set (checks my reading of the loops)
+        for m_idx in (0, 1, 7, 15, 16, 17, 31, 32, 40, 47):
+            lm, ll, la = _literal_stage1_block(Q[0, h], K[0, 0], V[0, 0], m_idx, SM)
+            rows = slice(m_idx * 128, (m_idx + 1) * 128)
+            np.testing.assert_allclose(lm, M[rows], atol=1e-9)
+            np.testing.assert_allclose(ll, L[rows], rtol=1e-9)
+            np.testing.assert_allclose(la, A[rows], rtol=1e-7, atol=1e-9)
+        # (b) the oracle agrees with the closed form: M to float32 dot accuracy, L/Acc to the
+        # bf16 rounding of p (relative 2^-9 per term)
+        np.testing.assert_allclose(res.M[0, h], M, atol=2e-5 * np.abs(M).max())
+        np.testing.assert_allclose(res.L[0, h], L, rtol=1e-5)
+        np.testing.assert_allclose(res.Acc[0, h] / res.L[0, h][:, None], A / L[:, None], atol=6e-3)
+
+
+def test_stage1_is_library_causal_attention_for_first_two_big_blocks():
+    q, k, v, _ = make_qkv(2 * S, 4, 2, n_stripes=32, seed=3)
+    Q, K, V = _np(q, k, v)
+    M, L, Acc = ao.stage1_anchor(Q, K, V, SM)
+    q1 = torch.from_numpy(ao.q1_scale_chain(Q, SM)) * math.log(2.0)
+    kk = torch.from_numpy(K).repeat_interleave(2, dim=1)
+    vv = torch.from_numpy(V).repeat_interleave(2, dim=1)
+    ref = torch.nn.functional.scaled_dot_product_attention(q1.double(), kk.double(), vv.double(), is_causal=True, scale=1.0)
+    got = Acc / L[..., None]
+    np.testing.assert_allclose(got, ref.numpy(), atol=6e-3)
+    assert np.abs(got - ref.numpy()).mean() < 3e-4
+    # the anchor is the row max of the scaled logits in the log2 domain
+    s = torch.einsum("bhnd,bhmd->bhnm", q1.double() / math.log(2.0), kk.double())
+    s = s.masked_fill(~torch.ones(2 * S, 2 * S, dtype=torch.bool).tril(), -float("inf"))
+    np.testing.assert_allclose(M, s.amax(-1).numpy(), atol=1e-3)
+
+
+def test_stage1_tile_width_only_changes_rounding(small):
+    Q, K, V, _, res = small
+    M2, L2, A2 = ao.stage1_anchor(Q[:, :1], K, V, SM, tile_n=64)
+    assert np.array_equal(M2[0, 0], res.M[0, 0])  # a max does not depend on tiling
+    np.testing.assert_allclose(L2[0, 0], res.L[0, 0], rtol=1e-5)
+    np.testing.assert_allclose(A2[0, 0] / L2[0, 0][:, None], res.Acc[0, 0] / res.L[0, 0][:, None], atol=4e-3)
+
+
+# ---------------------------------------------------------------- stage 2
+def test_stage2_structure_and_closed_forms(small):
+    Q, K, V, pos, res = small
+    n_bb = Q.shape[2] // S
+    for h in range(2):
+        assert res.counts[0, h, 0] == 0 and res.coords[0][h][0].size == 0
+        for bb in range(1, n_bb):
+            c = res.coords[0][h][bb]
+            assert c.dtype == np.int32 and c.size == res.counts[0, h, bb]
+            assert np.all(np.diff(c) > 0)
+            if c.size:
+                assert c[0] >= 128 and c[-1] < bb * S - 128
+    # theta -> +inf: every candidate; theta -> -inf: none; monotone in theta
+    allc, alln = ao.stage2_select(Q, K, res.M, SM, 1e4)
+    for bb in range(n_bb):
+        want = np.arange(128, bb * S - 128, dtype=np.int32) if bb else np.zeros(0, np.int32)
+        assert np.array_equal(allc[0][1][bb], want)
+        assert alln[0, 1, bb] == max(bb * S - 256, 0)
+    _, none = ao.stage2_select(Q, K, res.M, SM, -1e4)
+    assert none.sum() == 0
+    prev = None
+    for theta in (8.0, 10.0, 12.0, 14.0, 16.0):
+        c, _ = ao.stage2_select(Q, K, res.M, SM, theta)
+        cur = [set(c[0][0][bb].tolist()) for bb in range(n_bb)]
+        if prev is not None:
+            assert all(a <= b for a, b in zip(prev, cur))
+        prev = cur
+    # on this input the stripes (and only keys carrying the stripe bias) are what gets picked
+    picked = set(np.concatenate(res.coords[0][0]).tolist())
+    assert picked and picked <= set(pos.tolist())
+
+
+def test_stage2_independent_bruteforce(small):
+    """Same decisions from an independent route: torch bf16 casts, float64 dots, dense boolean
+    matrix, then the candidate slice - in the style of the reference's own torch restatement
+    get_mask_block (get_mask_test.py:162-232) plus the kernel's rounding points."""
+    Q, K, V, pos, res = small
+    N = Q.shape[2]
+    theta = 12.0
+    diff = torch.tensor(theta * ao.LOG2E, dtype=torch.float32)
+    for h in range(2):
+        q = torch.from_numpy(Q[0, h])
+        qbar = (q.view(N // 128, 128, D).double().sum(1) / 128).float().to(torch.bfloat16)
+        abar = (torch.from_numpy(res.M[0, h]).view(N // 128, 128).double().sum(1) / 128).float().to(torch.bfloat16)
+        raw = (qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (SM * ao.LOG2E)
+        sc = raw.float().to(torch.bfloat16)
+        hit = (sc.float() + diff) >= abar.float()[:, None]  # [N/128, N]
+        big = hit.view(N // S, 16, N).any(1)
+        for bb in range(N // S):
+            want = torch.nonzero(big[bb, 128 : max(bb * S - 128, 128)])[:, 0] + 128
+            got = res.coords[0][h][bb]
+            sym = set(want.tolist()) ^ set(got.tolist())
+            # float64-vs-float32 dots may only disagree right at a decision boundary
+            for j in sym:
+                rows = slice(bb * 16, bb * 16 + 16)
+                ab, mean = ao.pooled_anchors(res.M[0, h], 128)
+                d = ao.stage2_flip_distance(ao.pooled_queries(Q[0, h], 128)[rows], ab[rows], mean[rows], K[0, 0, j], SM, theta)
+                assert d < 1e-3
+            assert len(sym) <= 2
+
+
+def test_stage2_decision_boundary_is_where_the_decision_flips():
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        abar = float(ao.rn16(np.array([rng.uniform(5, 40)], np.float32))[0])
+        theta = float(rng.uniform(6, 18))
+        diff = np.float32(theta * ao.LOG2E)
+        b = ao.stage2_decision_boundary(abar, theta)
+        for eps, want in ((+1e-4, True), (-1e-4, False)):
+            sc = ao.rn16(np.array([b + eps], np.float32))[0]
+            assert bool(np.float32(sc + diff) >= np.float32(abar)) is want
+
+
+# ---------------------------------------------------------------- stage 3 and the whole operator
+def test_stage3_multiplicity_closed_form(small):
+    """out_r = sum_j c_j 2^{s_rj} v_j / sum_j c_j 2^{s_rj}; c_j = [j in W(r)] + [j in Sel(bb)];
+    window logits use the stage-1 scaling, stripe logits the stage-3 scaling."""
+    Q, K, V, pos, res = small
+    N = Q.shape[2]
+    wmask = _window_mask(N)
+    k64, v64 = K[0, 0].astype(np.float64), V[0, 0].astype(np.float64)
+    for h in range(2):
+        s1 = ao.q1_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        s3 = ao.q3_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        sel = np.zeros((N, N), bool)
+        for bb in range(N // S):
+            sel[bb * S : (bb + 1) * S, res.coords[0][h][bb]] = True
+        s1 = np.where(wmask, s1, -np.inf)
+        s3 = np.where(sel, s3, -np.inf)
+        mx = np.maximum(s1.max(1), s3.max(1))
+        w = np.exp2(s1 - mx[:, None]) + np.exp2(s3 - mx[:, None])
+        want = (w @ v64) / w.sum(1)[:, None]
+        err = np.abs(res.out[0, h] - want)
+        assert err.max() < 2e-2 and err.mean() < 1.5e-3
+        # the double count matters: leaving it out must break the tolerance on this input
+        sel_nodup = sel & ~wmask
+        w2 = np.exp2(s1 - mx[:, None]) + np.exp2(np.where(sel_nodup, s3, -np.inf) - mx[:, None])
+        assert np.abs((w2 @ v64) / w2.sum(1)[:, None] - res.out[0, h]).max() > 5e-2
+    assert (sel & wmask).any()
+
+
+def test_stage3_constant_values_give_that_value(small):
+    Q, K, V, pos, res = small
+    row = ao.rn16(np.linspace(-2, 2, D).astype(np.float32))
+    Vc = np.broadcast_to(row, V.shape).copy()
+    out = ao.anchor_attn_reference(Q, K, Vc, difference=12.0).out
+    np.testing.assert_allclose(out, np.broadcast_to(row, out.shape), atol=2e-2, rtol=1e-2)
+
+
+def test_theta_minus_inf_at_two_big_blocks_is_dense_causal_attention():
+    q, k, v, _ = make_qkv(2 * S, 2, 2, n_stripes=32, seed=5)
+    Q, K, V = _np(q, k, v)
+    res = ao.anchor_attn_reference(Q, K, V, difference=-1e4)
+    assert res.counts.sum() == 0 and res.ratio == 0.0
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(Q).double(), torch.from_numpy(K).double(), torch.from_numpy(V).double(), is_causal=True
+    ).numpy()
+    err = np.abs(res.out - ref)
+    # stage-1 scale chain inflates logits by 1.0017: allow for it
+    assert err.max() < 3e-2 and err.mean() < 2e-3
+
+
+def test_ratio_formula_and_gap(small):
+    Q, K, V, pos, res = small
+    B, H, N, _ = Q.shape
+    assert res.ratio == res.counts.sum() / math.floor(B * H * N * N / 2048 / 2)
+    assert ao.sparsity_ratio(np.array([[[0, 1792]]]), 1, 1, 4096, 128, 16) == 1792 / 4096.0
+    # keys in [bb*S-128, bb*S) are never candidates for bb >= 2
+    allc, _ = ao.stage2_select(Q, K, res.M, SM, 1e4)
+    assert allc[0][0][2].max() == 2 * S - 129
+
+
+def test_reference_layout_packing(small):
+    Q, K, V, pos, res = small
+    tc = ao.coords_to_reference_layout(res.coords, res.counts, Q.shape[2])
+    assert tc.shape == (1, 2, 3, Q.shape[2]) and tc.dtype == np.int32
+    c = res.coords[0][1][2]
+    assert np.array_equal(tc[0, 1, 2, : c.size], c) and not tc[0, 1, 2, c.size :].any()
