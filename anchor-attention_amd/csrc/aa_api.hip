@@ -1,0 +1,334 @@
+// C ABI of the AnchorAttention gfx950 kernels: argument validation, scratch carving, launches.
+// Declarations and their reference counterparts: include/anchor_attn_hip.h.
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/anchor_attn_hip.h"
+#include "aa_common.h"
+#include "aa_kernels.h"
+
+namespace aa {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+namespace {
+
+struct Dims {
+  int batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step;
+};
+
+int check_dims(const Dims& d, const char* who) {
+  if (d.batch <= 0 || d.n_q_heads <= 0 || d.n_kv_heads <= 0 || d.n_ctx <= 0) {
+    set_error("%s: batch, head counts and n_ctx must be positive (got %d, %d, %d, %d)", who, d.batch, d.n_q_heads, d.n_kv_heads, d.n_ctx);
+    return AA_EBADARG;
+  }
+  if (d.n_q_heads % d.n_kv_heads != 0) {
+    set_error("%s: n_kv_heads (%d) must divide n_q_heads (%d)", who, d.n_kv_heads, d.n_q_heads);
+    return AA_EBADARG;
+  }
+  if (d.head_dim != 128) {
+    set_error("%s: head_dim %d is not supported (only 128)", who, d.head_dim);
+    return AA_EUNSUPPORTED;
+  }
+  if (d.block_size != 128) {
+    set_error("%s: block_size %d is not supported (only 128)", who, d.block_size);
+    return AA_EUNSUPPORTED;
+  }
+  if (d.step != 16 && d.step != 32) {
+    set_error("%s: step %d is not supported (16 or 32)", who, d.step);
+    return AA_EUNSUPPORTED;
+  }
+  if (d.n_ctx % (d.block_size * d.step) != 0) {
+    set_error("%s: n_ctx %d is not a multiple of block_size*step = %d", who, d.n_ctx, d.block_size * d.step);
+    return AA_EUNSUPPORTED;
+  }
+  if ((int64_t)d.batch * d.n_q_heads * (d.n_ctx / 128) > 0x7fffffffLL) {
+    set_error("%s: problem too large for one launch", who);
+    return AA_EUNSUPPORTED;
+  }
+  return AA_OK;
+}
+
+int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, const char* who, const char* name) {
+  if (ptr == nullptr) {
+    set_error("%s: %s is NULL", who, name);
+    return AA_EBADARG;
+  }
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15u) != 0 || (sb % 8) != 0 || (sh % 8) != 0 || (sn % 8) != 0) {
+    set_error("%s: %s must be 16-byte aligned with strides that are multiples of 8 elements (ptr=%p strides=%lld,%lld,%lld)", who, name, ptr, (long long)sb, (long long)sh, (long long)sn);
+    return AA_EMISALIGNED;
+  }
+  if (sn < 128) {
+    set_error("%s: %s row stride %lld is smaller than head_dim", who, name, (long long)sn);
+    return AA_EBADARG;
+  }
+  return AA_OK;
+}
+
+int check_ptr(const void* ptr, const char* who, const char* name) {
+  if (ptr == nullptr) {
+    set_error("%s: %s is NULL", who, name);
+    return AA_EBADARG;
+  }
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15u) != 0) {
+    set_error("%s: %s must be 16-byte aligned", who, name);
+    return AA_EMISALIGNED;
+  }
+  return AA_OK;
+}
+
+int check_launch(hipError_t e, const char* who) {
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", who, hipGetErrorString(e));
+    return AA_ELAUNCH;
+  }
+  return AA_OK;
+}
+
+// query rows per work-group = 128 * qb; 2 unless AA_FLASH_QB=1 is exported (tuning knob)
+int flash_qb() {
+  static const int qb = [] {
+    const char* e = getenv("AA_FLASH_QB");
+    return (e && e[0] == '1') ? 1 : 2;
+  }();
+  return qb;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+struct Workspace {
+  size_t M, L, acc, qbar, abar, mask, coords, counts, total;
+};
+
+Workspace carve(int batch, int hq, int n_ctx, int block_size, int step) {
+  Workspace w;
+  const size_t bh = (size_t)batch * hq;
+  size_t off = 0;
+  w.M = off;      off += align256(bh * n_ctx * 4);
+  w.L = off;      off += align256(bh * n_ctx * 4);
+  w.acc = off;    off += align256(bh * n_ctx * 128 * 4);
+  w.qbar = off;   off += align256(bh * (n_ctx / block_size) * 128 * 2);
+  w.abar = off;   off += align256(bh * (n_ctx / block_size) * 2);
+  w.mask = off;   off += align256((size_t)aa_mask_words(batch, hq, n_ctx, block_size, step) * 4);
+  w.coords = off; off += align256(bh * (size_t)aa_coords_entries_per_head(n_ctx, block_size, step) * 4);
+  w.counts = off; off += align256(bh * (n_ctx / (block_size * step)) * 4);
+  w.total = off;
+  return w;
+}
+
+}  // namespace
+}  // namespace aa
+
+using namespace aa;
+
+extern "C" {
+
+int aa_version(void) { return 1; }
+
+const char* aa_last_error(void) { return g_error; }
+
+int64_t aa_coords_entries_per_head(int n_ctx, int block_size, int step) {
+  const int64_t S = (int64_t)block_size * step;
+  return coords_tri(n_ctx / S, S, block_size);
+}
+
+int64_t aa_coords_offset(int big_block, int block_size, int step) {
+  return coords_tri(big_block, (int64_t)block_size * step, block_size);
+}
+
+int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int step) {
+  return (int64_t)batch * n_q_heads * (n_ctx / (block_size * step)) * (n_ctx / 128) * 4;
+}
+
+size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int step) {
+  if (batch <= 0 || n_q_heads <= 0 || n_ctx <= 0 || head_dim != 128 || block_size <= 0 || step <= 0) return 0;
+  return carve(batch, n_q_heads, n_ctx, block_size, step).total;
+}
+
+int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         float* M, float* L, float* acc_frag,
+                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                         int block_size, int step, float sm_scale, int scale_mode, void* stream) {
+  const char* who = "aa_stage1_anchor_fwd";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
+  if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag"))) return rc;
+  if (scale_mode != AA_SCALE_BF16_CHAIN && scale_mode != AA_SCALE_FP32) {
+    set_error("%s: unknown scale_mode %d", who, scale_mode);
+    return AA_EBADARG;
+  }
+  FlashArgs a = {};
+  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.M_out = M; a.L_out = L; a.acc_out = acc_frag;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.big_block = block_size * step; a.block_size = block_size;
+  a.sm_scale = sm_scale; a.scale_mode = scale_mode;
+  return check_launch(launch_flash(a, 0, flash_qb(), (hipStream_t)stream), who);
+}
+
+int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
+                     void* qbar, void* abar,
+                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, void* stream) {
+  const char* who = "aa_pool_q_anchor";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_q_heads, n_ctx, head_dim, block_size, 16}, who))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
+  if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar"))) return rc;
+  PoolArgs a = {};
+  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.M = M; a.qbar = (__bf16*)qbar; a.abar = (__bf16*)abar;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_ctx = n_ctx; a.block_size = block_size;
+  return check_launch(launch_pool(a, (hipStream_t)stream), who);
+}
+
+int aa_stage2_select(const void* qbar, const void* abar,
+                     const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                     uint32_t* mask_ws, int32_t* coords, int32_t* counts,
+                     int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                     int block_size, int step, float sm_scale, float theta_log2, void* stream) {
+  const char* who = "aa_stage2_select";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
+  if ((rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar")) || (rc = check_ptr(mask_ws, who, "mask_ws")) ||
+      (rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")))
+    return rc;
+  SelectArgs a = {};
+  a.qbar = (const __bf16*)qbar; a.abar = (const __bf16*)abar;
+  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.mask = mask_ws; a.coords = coords; a.counts = counts;
+  a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.big_block = block_size * step; a.block_size = block_size;
+  a.scale2 = (float)((double)sm_scale * 1.44269504);  // double product, then float32, as the definition does
+  a.theta_log2 = theta_log2;
+  if ((rc = check_launch(launch_select_scores(a, (hipStream_t)stream), who))) return rc;
+  return check_launch(launch_select_compact(a, (hipStream_t)stream), who);
+}
+
+int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         const int32_t* coords, const int32_t* counts,
+                         const float* M, const float* L, const float* acc_frag,
+                         void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                         int block_size, int step, float sm_scale, void* stream) {
+  const char* who = "aa_stage3_sparse_fwd";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, who, "out"))) return rc;
+  if ((rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")) || (rc = check_ptr(M, who, "M")) ||
+      (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag")))
+    return rc;
+  FlashArgs a = {};
+  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.out = (__bf16*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.M = M; a.L = L; a.acc_frag = acc_frag;
+  a.coords = coords; a.counts = counts;
+  a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.big_block = block_size * step; a.block_size = block_size;
+  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
+  return check_launch(launch_flash(a, 1, flash_qb(), (hipStream_t)stream), who);
+}
+
+int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                       const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                       const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                       void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                       void* workspace, size_t workspace_bytes, int32_t* counts_out,
+                       int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                       int block_size, int step, float sm_scale, float theta, int scale_mode,
+                       void* stream) {
+  const char* who = "aa_anchor_attn_fwd";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  if ((rc = check_ptr(workspace, who, "workspace"))) return rc;
+  const Workspace w = carve(batch, n_q_heads, n_ctx, block_size, step);
+  if (workspace_bytes < w.total) {
+    set_error("%s: workspace has %zu bytes, %zu needed", who, workspace_bytes, w.total);
+    return AA_EBADARG;
+  }
+  char* ws = static_cast<char*>(workspace);
+  float* M = (float*)(ws + w.M);
+  float* L = (float*)(ws + w.L);
+  float* acc = (float*)(ws + w.acc);
+  void* qbar = ws + w.qbar;
+  void* abar = ws + w.abar;
+  uint32_t* mask = (uint32_t*)(ws + w.mask);
+  int32_t* coords = (int32_t*)(ws + w.coords);
+  int32_t* counts = (int32_t*)(ws + w.counts);
+  if ((rc = aa_stage1_anchor_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc, batch, n_q_heads,
+                                 n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, scale_mode, stream)))
+    return rc;
+  if ((rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, stream))) return rc;
+  // theta -> log2 domain: a double product rounded to float32 (the definition multiplies a Python float)
+  const float theta_log2 = (float)((double)theta * 1.44269504);
+  if ((rc = aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, mask, coords, counts, batch, n_q_heads, n_kv_heads, n_ctx,
+                             head_dim, block_size, step, sm_scale, theta_log2, stream)))
+    return rc;
+  if ((rc = aa_stage3_sparse_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, coords, counts, M, L, acc, out,
+                                 o_sb, o_sh, o_sn, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale,
+                                 stream)))
+    return rc;
+  if (counts_out != nullptr) {
+    const size_t bytes = (size_t)batch * n_q_heads * (n_ctx / (block_size * step)) * 4;
+    hipError_t e = hipMemcpyAsync(counts_out, counts, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream);
+    if ((rc = check_launch(e, who))) return rc;
+  }
+  return AA_OK;
+}
+
+int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                        const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                        float sm_scale, void* stream) {
+  const char* who = "aa_dense_causal_fwd";
+  int rc;
+  if (n_ctx <= 0 || n_ctx % 256 != 0) {
+    set_error("%s: n_ctx %d must be a positive multiple of 256", who, n_ctx);
+    return AA_EUNSUPPORTED;
+  }
+  Dims d = {batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16};
+  d.n_ctx = 2048;  // only the generic checks; divisibility by the big block does not apply here
+  if ((rc = check_dims(d, who))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, who, "out"))) return rc;
+  FlashArgs a = {};
+  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.out = (__bf16*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.big_block = n_ctx; a.block_size = 128;  // one "big block": bb is always 0
+  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
+  return check_launch(launch_flash(a, 2, flash_qb(), (hipStream_t)stream), who);
+}
+
+}  // extern "C"

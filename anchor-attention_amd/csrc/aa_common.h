@@ -1,0 +1,59 @@
+// Shared device/host helpers for the AnchorAttention gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.44269504f;  // the literal the operator's definition multiplies by
+
+// ---- bf16 <-> float -------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
+// round-to-nearest-even float -> bf16, two at a time (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  floatx2 f = {a, b};
+  bf16x2 h = __builtin_convertvector(f, bf16x2);
+  return *reinterpret_cast<uint32_t*>(&h);
+}
+// float -> nearest bf16 -> float
+__device__ __forceinline__ float rn16(float a) { return bf16_lo(pack_bf16(a, 0.f)); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// value held by the lane 32 positions away (the two halves of a wave share MFMA columns)
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// ---- geometry --------------------------------------------------------------------------------
+// Index lists are packed per (batch, query head): big block bb can select at most
+// cap(bb) = bb*S - 2*bs keys (candidates are [bs, bb*S - bs)), and its list starts at
+// tri(bb) = sum_{x<bb} cap(x) entries into the head's slab.
+__host__ __device__ inline int64_t coords_tri(int64_t bb, int64_t S, int64_t bs) {
+  return bb <= 1 ? 0 : S * (bb - 1) * bb / 2 - 2 * bs * (bb - 1);
+}
+
+// XCD-aware work-group renumbering: consecutive hardware work-group ids go round-robin over the
+// 8 XCDs (each with its own L2); give every XCD one contiguous range of logical ids so that
+// neighbours in the logical order (which share K/V tiles) hit the same L2.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t total) {
+  return (total % 8u == 0u) ? (wg % 8u) * (total / 8u) + wg / 8u : wg;
+}
+
+// ---- error plumbing (host) -------------------------------------------------------------------
+enum Status : int {
+  kOk = 0,
+  kBadArgument = 1,   // null pointer, non-positive size, inconsistent head counts
+  kUnsupported = 2,   // a size the kernels are not written for (head_dim, block_size, step)
+  kMisaligned = 3,    // pointer or stride breaks the 16-byte row alignment the loads assume
+  kLaunchFailed = 4,  // the HIP runtime refused the launch
+};
+void set_error(const char* fmt, ...);
+
+}  // namespace aa

@@ -1,0 +1,42 @@
+// Internal launch interfaces between the C-ABI layer and the kernel translation units.
+#pragma once
+#include "aa_common.h"
+
+namespace aa {
+
+struct FlashArgs {
+  const __bf16* q; int64_t q_sb, q_sh, q_sn;
+  const __bf16* k; int64_t k_sb, k_sh, k_sn;
+  const __bf16* v; int64_t v_sb, v_sh, v_sn;
+  __bf16* out;     int64_t o_sb, o_sh, o_sn;   // sparse / dense modes
+  float* M_out; float* L_out; float* acc_out;  // anchor mode
+  const float* M; const float* L; const float* acc_frag;  // sparse mode (resume state)
+  const int32_t* coords; const int32_t* counts; int64_t coords_per_head;  // sparse mode
+  int batch, n_q_heads, n_kv_heads, n_ctx;
+  int big_block, block_size;
+  float sm_scale; int scale_mode;
+};
+
+// mode: 0 anchor (stage 1), 1 sparse (stage 3), 2 dense causal.  qb: 32-row query blocks per wave (1|2).
+hipError_t launch_flash(const FlashArgs& a, int mode, int qb, hipStream_t stream);
+
+struct PoolArgs {
+  const __bf16* q; int64_t q_sb, q_sh, q_sn;
+  const float* M;
+  __bf16* qbar; __bf16* abar;
+  int batch, n_q_heads, n_ctx, block_size;
+};
+hipError_t launch_pool(const PoolArgs& a, hipStream_t stream);
+
+struct SelectArgs {
+  const __bf16* qbar; const __bf16* abar;
+  const __bf16* k; int64_t k_sb, k_sh, k_sn;
+  uint32_t* mask; int32_t* coords; int32_t* counts; int64_t coords_per_head;
+  int batch, n_q_heads, n_kv_heads, n_ctx;
+  int big_block, block_size;
+  float scale2, theta_log2;
+};
+hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream);
+hipError_t launch_select_compact(const SelectArgs& a, hipStream_t stream);
+
+}  // namespace aa

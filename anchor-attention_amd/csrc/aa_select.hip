@@ -1,0 +1,202 @@
+// Stage 2 of the AnchorAttention prefill path on gfx950: pooling, score-and-threshold, compaction.
+//
+//  pool     qbar = bf16(mean of 128 raw query rows), abar = bf16(mean of 128 anchors); float32 sums in
+//           ascending row order so the result is reproducible bit for bit.
+//  scores   K-stationary: one work-group per (batch, KV head, 128-key tile) keeps the key tile in
+//           registers as the MFMA B operand and streams the pooled query rows of EVERY query head of
+//           the KV group and EVERY later big block past it (A operand, 32 pooled rows per MFMA).  Each
+//           K row is thus read once per KV head instead of once per (query head, big block).
+//           In the 32x32 accumulator a lane holds one key column; OR-ing its registers over the pooled
+//           rows of a big block and a wave ballot give a 32-bit key mask per (q head, big block, key
+//           block) with no LDS and no atomics.
+//  compact  one wave per (batch, q head, big block) turns that big block's mask row into an ascending
+//           index list with popcounts and a wave prefix sum.
+#include "aa_common.h"
+#include "aa_kernels.h"
+
+namespace aa {
+
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
+  const int lane = threadIdx.x;
+  const int c = lane & 15;
+  const int n_pr = p.n_ctx / p.block_size;
+  const int pr = 4 * blockIdx.x + (lane >> 4);
+  const int h = blockIdx.y, b = blockIdx.z;
+  if (pr >= n_pr) return;
+  const int bs = p.block_size;
+  const __bf16* base = p.q + b * p.q_sb + h * p.q_sh + (int64_t)pr * bs * p.q_sn + 8 * c;
+  const int64_t bh = (int64_t)b * p.n_q_heads + h;
+  const float* mb = p.M + bh * p.n_ctx + (int64_t)pr * bs;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float am = 0.f;
+#pragma unroll 8
+  for (int t = 0; t < bs; ++t) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(base + (int64_t)t * p.q_sn);
+    acc[0] += bf16_lo(raw.x); acc[1] += bf16_hi(raw.x);
+    acc[2] += bf16_lo(raw.y); acc[3] += bf16_hi(raw.y);
+    acc[4] += bf16_lo(raw.z); acc[5] += bf16_hi(raw.z);
+    acc[6] += bf16_lo(raw.w); acc[7] += bf16_hi(raw.w);
+    if (c == 0) am += mb[t];
+  }
+  const float d = (float)bs;
+  uint4 o;
+  o.x = pack_bf16(acc[0] / d, acc[1] / d);
+  o.y = pack_bf16(acc[2] / d, acc[3] / d);
+  o.z = pack_bf16(acc[4] / d, acc[5] / d);
+  o.w = pack_bf16(acc[6] / d, acc[7] / d);
+  *reinterpret_cast<uint4*>(p.qbar + (bh * n_pr + pr) * 128 + 8 * c) = o;
+  if (c == 0) {
+    const uint32_t w = pack_bf16(am / d, 0.f);
+    reinterpret_cast<uint16_t*>(p.abar)[bh * n_pr + pr] = (uint16_t)(w & 0xffffu);
+  }
+}
+
+hipError_t launch_pool(const PoolArgs& a, hipStream_t stream) {
+  const int n_pr = a.n_ctx / a.block_size;
+  hipLaunchKernelGGL(pool_kernel, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+// STEP = pooled rows per big block (16 or 32); 32 / STEP (head, big block) items share one MFMA.
+template <int STEP>
+__global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) {
+  constexpr int kItems = 32 / STEP;
+  const int t = blockIdx.x;  // key tile (128 keys)
+  const int kvh = blockIdx.y, b = blockIdx.z;
+  const int n_bb = p.n_ctx / p.big_block;
+  const int n_t = p.n_ctx / 128;
+  const int n_pr = n_t;  // pooled rows per head (block_size == 128)
+  // tile t is a candidate for big block bb iff 1 <= t <= STEP*bb - 2
+  if (t == 0) return;
+  const int bb_min = (t + 2 + STEP - 1) / STEP;
+  if (bb_min >= n_bb) return;
+  const int group = p.n_q_heads / p.n_kv_heads;
+  const int n_items = group * (n_bb - bb_min);
+  const int n_groups = (n_items + kItems - 1) / kItems;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, c32 = lane & 31;
+
+  const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
+  bf16x8 kreg[4][8];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    const __bf16* row = kp + (int64_t)(t * 128 + 32 * kb + c32) * p.k_sn + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
+  }
+
+  for (int grp = wave; grp < n_groups; grp += 4) {
+    // A operand: row c32 of this MFMA is pooled row (c32 % STEP) of item grp*kItems + c32/STEP
+    const int item_a = min(grp * kItems + c32 / STEP, n_items - 1);
+    const int hq_a = kvh * group + item_a % group;
+    const int bb_a = bb_min + item_a / group;
+    const __bf16* qrow = p.qbar + (((int64_t)b * p.n_q_heads + hq_a) * n_pr + bb_a * STEP + c32 % STEP) * 128 + 8 * half;
+    bf16x8 a[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks);
+
+    // thresholds for the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
+    float thr[16];
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const int i0 = 8 * rq + 4 * half;
+      const int item = min(grp * kItems + i0 / STEP, n_items - 1);
+      const int hq = kvh * group + item % group;
+      const int bb = bb_min + item / group;
+      const uint2 w = *reinterpret_cast<const uint2*>(p.abar + ((int64_t)b * p.n_q_heads + hq) * n_pr + bb * STEP + i0 % STEP);
+      thr[4 * rq + 0] = bf16_lo(w.x); thr[4 * rq + 1] = bf16_hi(w.x);
+      thr[4 * rq + 2] = bf16_lo(w.y); thr[4 * rq + 3] = bf16_hi(w.y);
+    }
+
+    uint32_t words[kItems][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      floatx16 c;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) c[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c, 0, 0, 0);
+      bool hit[kItems];
+#pragma unroll
+      for (int it = 0; it < kItems; ++it) hit[it] = false;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float sc = rn16(c[r] * p.scale2);          // float32 product, then bf16
+        const bool pass = (sc + p.theta_log2) >= thr[r];  // float32 add and compare, non-strict
+        hit[(8 * (r >> 2)) / STEP] |= pass;                // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
+      }
+#pragma unroll
+      for (int it = 0; it < kItems; ++it) {
+        const uint64_t m = __ballot(hit[it]);
+        words[it][kb] = (uint32_t)m | (uint32_t)(m >> 32);  // both halves of the wave hold the same keys
+      }
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int it = 0; it < kItems; ++it) {
+        const int item = grp * kItems + it;
+        if (item < n_items) {
+          const int hq = kvh * group + item % group;
+          const int bb = bb_min + item / group;
+          uint4 w = {words[it][0], words[it][1], words[it][2], words[it][3]};
+          *reinterpret_cast<uint4*>(p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + t) * 4) = w;
+        }
+      }
+    }
+  }
+}
+
+hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
+  const int step = a.big_block / a.block_size;
+  const dim3 grid(a.n_ctx / 128, a.n_kv_heads, a.batch);
+  if (step == 16) hipLaunchKernelGGL(select_scores_kernel<16>, grid, dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(select_scores_kernel<32>, grid, dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(64) select_compact_kernel(const SelectArgs p) {
+  const int bb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x;
+  const int n_bb = p.n_ctx / p.big_block;
+  const int n_t = p.n_ctx / 128;
+  const int step = p.big_block / p.block_size;
+  const int64_t bh = (int64_t)b * p.n_q_heads + h;
+  const int t_lo = 1, t_hi = step * bb - 2;  // candidate key tiles, inclusive
+  int base = 0;
+  if (t_hi >= t_lo) {
+    const int n_words = 4 * (t_hi - t_lo + 1);
+    const uint32_t* mw = p.mask + ((bh * n_bb + bb) * n_t + t_lo) * 4;
+    int32_t* out = p.coords + bh * p.coords_per_head + coords_tri(bb, p.big_block, p.block_size);
+    for (int w0 = 0; w0 < n_words; w0 += 64) {
+      const int wi = w0 + lane;
+      uint32_t word = wi < n_words ? mw[wi] : 0u;
+      const int pc = __popc(word);
+      int incl = pc;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+      }
+      int pos = base + incl - pc;
+      const int key_base = t_lo * 128 + wi * 32;
+      while (word) {
+        out[pos++] = key_base + (__ffs(word) - 1);
+        word &= word - 1;
+      }
+      base += __shfl(incl, 63, 64);
+    }
+  }
+  if (lane == 0) p.counts[bh * n_bb + bb] = base;
+}
+
+hipError_t launch_select_compact(const SelectArgs& a, hipStream_t stream) {
+  hipLaunchKernelGGL(select_compact_kernel, dim3(a.n_ctx / a.big_block, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace aa

@@ -1,0 +1,141 @@
+/*
+ * anchor_attn_hip.h - C ABI of the gfx950 (MI355X) AnchorAttention prefill kernels.
+ *
+ * Every entry point takes plain device pointers, sizes, element strides and a HIP stream
+ * (passed as void*; NULL is the default stream).  The library never allocates or frees device
+ * memory: scratch is handed in by the caller.  All launches are asynchronous on the given
+ * stream and nothing synchronises the device.  Return value: 0 on success, otherwise one of
+ * the AA_E* codes; aa_last_error() then describes the failure (thread-local string).
+ *
+ * Tensors: q/out are [batch, n_q_heads, n_ctx, head_dim]; k/v are [batch, n_kv_heads, n_ctx,
+ * head_dim] with n_kv_heads dividing n_q_heads (query head h reads KV head
+ * h / (n_q_heads / n_kv_heads), the order repeat_kv produces; pass n_kv_heads == n_q_heads for
+ * pre-repeated K/V as the reference's caller does).  Element type is bf16, head_dim must be
+ * 128 with stride 1, every row must start on a 16-byte boundary; the other three dimensions
+ * are addressed through the element strides (sb, sh, sn), so [B,N,H,D] storage works unchanged.
+ * "S" below is the big block, block_size * step keys/queries.
+ *
+ * Reference citations are paths inside yuzhouzhang9/Anchor-Attention.
+ */
+#ifndef ANCHOR_ATTN_HIP_H_
+#define ANCHOR_ATTN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AA_OK 0
+#define AA_EBADARG 1      /* null pointer, non-positive size, head counts that do not divide */
+#define AA_EUNSUPPORTED 2 /* head_dim != 128, block_size != 128, step not 16/32, n_ctx % S != 0 */
+#define AA_EMISALIGNED 3  /* pointer or stride not a multiple of 16 bytes */
+#define AA_ELAUNCH 4      /* HIP runtime error at launch */
+
+/* How stage 1 pre-scales queries.  AA_SCALE_BF16_CHAIN reproduces the reference's stage-1
+ * kernel, where sm_scale is a compile-time constant and q * sm_scale * 1.44269504 is therefore
+ * evaluated in bf16 with a rounding after each multiply (anchor_step_1_2_v2.py:19,115-116).
+ * AA_SCALE_FP32 is the float32 product rounded once (what stage 3 does, anchor_attn_v4.py:66). */
+#define AA_SCALE_BF16_CHAIN 0
+#define AA_SCALE_FP32 1
+
+int aa_version(void);
+const char* aa_last_error(void);
+
+/* ---- scratch geometry ---------------------------------------------------------------------- */
+
+/* Selected-key index lists are packed: per (batch, q head) one slab of
+ * aa_coords_entries_per_head() int32; big block bb's ascending list starts at
+ * aa_coords_offset(bb) inside the slab and holds counts[b,h,bb] entries (capacity
+ * bb*S - 2*block_size, the number of candidate keys).  Replaces the reference's
+ * true_coords [B,H,N/S,N] buffer (get_mask_test.py:138-141). */
+int64_t aa_coords_entries_per_head(int n_ctx, int block_size, int step);
+int64_t aa_coords_offset(int big_block, int block_size, int step);
+
+/* Number of uint32 words of the stage-2 key bitmask: [batch, n_q_heads, n_ctx/S, n_ctx/128, 4]. */
+int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int step);
+
+/* Bytes of scratch aa_anchor_attn_fwd() needs (M, L, Acc, pooled q, pooled anchors, bitmask,
+ * index lists, counts - in that order, each 256-byte aligned). */
+size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int step);
+
+/* ---- stage 1: pattern-based anchor computation ---------------------------------------------
+ * Replaces anchor_attn_step_1 / get_mask_fused_anchor_triton with init_cnt = local_cnt = 1
+ * (anchor_step_1_2_v2.py:8-196; call site anchor_attn_v4.py:237-241): flash attention of each
+ * query row r over keys [0,S) U [bb*S, r] (bb = r / S), exp2 domain.
+ * Outputs: M [B,Hq,N] float32 running max (the anchors), L [B,Hq,N] float32 row sums,
+ * acc_frag float32 with B*Hq*N*128 elements: the unnormalised PV accumulator in MFMA fragment
+ * order - element (b,h,row,d) lives at ((((b*Hq+h)*(N/32) + row/32)*4 + d/32)*4 + (d%32)/8)*256
+ * + (((d%8)/4)*32 + row%32)*4 + d%4.  Stage 3 consumes exactly this order. */
+int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         float* M, float* L, float* acc_frag,
+                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                         int block_size, int step, float sm_scale, int scale_mode, void* stream);
+
+/* ---- stage 2: difference-aware stripe identification -------------------------------------- */
+
+/* Mean-pools raw queries and anchors over block_size rows, rounding to bf16
+ * (get_mask_test.py:75-84): qbar [B,Hq,N/block_size,128] bf16, abar [B,Hq,N/block_size] bf16.
+ * Sums run in float32 in ascending row order. */
+int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
+                     void* qbar, void* abar,
+                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, void* stream);
+
+/* Replaces anchor_attn_step_2 / get_q_mask / get_q_mask_triton (anchor_step_1_2_v2.py:199-210,
+ * get_mask_test.py:7-159): key j in [block_size, bb*S - block_size) is selected for big block bb
+ * iff for one of its pooled rows i  float(bf16(dot(qbar_i,k_j) * sm_scale*1.44269504)) + theta_log2
+ * >= float(abar_i).  theta_log2 is theta * 1.44269504 (anchor_attn_v4.py:298).
+ * mask_ws: scratch of aa_mask_words() uint32.  Outputs: coords (packed, see above) and
+ * counts [B,Hq,N/S] int32.  Deterministic: no atomics, lists are ascending. */
+int aa_stage2_select(const void* qbar, const void* abar,
+                     const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                     uint32_t* mask_ws, int32_t* coords, int32_t* counts,
+                     int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                     int block_size, int step, float sm_scale, float theta_log2, void* stream);
+
+/* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
+ * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
+ * :246-268): resumes the online softmax from (M, L, acc_frag) over the K/V rows gathered at the
+ * big block's selected indices and writes out = bf16(acc / l).  M, L, acc_frag are read-only. */
+int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         const int32_t* coords, const int32_t* counts,
+                         const float* M, const float* L, const float* acc_frag,
+                         void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                         int block_size, int step, float sm_scale, void* stream);
+
+/* ---- whole operator -------------------------------------------------------------------------
+ * Replaces _anchor_attn (anchor_attn_v4.py:226-273): stage 1 -> pooling -> stage 2 -> stage 3 on
+ * one stream.  workspace: aa_workspace_bytes() bytes of device scratch (contents undefined
+ * afterwards).  counts_out (optional, may be NULL): [B,Hq,N/S] int32 copy of the per-big-block
+ * selection counts, from which the caller forms the sparsity ratio (anchor_attn_v4.py:270-272).
+ * theta is in natural-log units as in the reference's `difference` argument. */
+int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                       const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                       const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                       void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                       void* workspace, size_t workspace_bytes, int32_t* counts_out,
+                       int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                       int block_size, int step, float sm_scale, float theta, int scale_mode,
+                       void* stream);
+
+/* ---- dense causal baseline on the same MFMA core --------------------------------------------
+ * Counterpart of the reference's dense comparison path (flash_attn_triton.py:83-211, GQA mapping
+ * :129-132): plain causal softmax attention, out = bf16(softmax(q k^T * sm_scale) v).
+ * n_ctx must be a multiple of 256. */
+int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                        const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                        float sm_scale, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ANCHOR_ATTN_HIP_H_ */

@@ -1,0 +1,302 @@
+"""GPU parity: the gfx950 kernels (through the C ABI) against the CPU oracle on the same seeded
+inputs.  Tolerances: index sets identical except keys whose pre-rounding score lies within 1e-3 of
+a decision flip; outputs max |err| <= 2e-2 and mean |err| <= 2e-3 (bf16)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D, BS, STEP, S = 128, 128, 16, 2048
+SM = 1.0 / math.sqrt(D)
+LOG2E = 1.44269504
+MAX_ERR, MEAN_ERR, BAND = 2e-2, 2e-3, 1e-3
+
+
+def _np(*ts):
+    return [t.float().cpu().numpy() for t in ts]
+
+
+@pytest.fixture(scope="module")
+def mods():
+    from anchor_attn.src.ops import _hip, anchor_attn_v4, anchor_step_1_2_v2
+    from oracle import anchor_oracle as ao
+    assert torch.cuda.is_available()
+    _hip.lib()
+    return _hip, anchor_attn_v4, anchor_step_1_2_v2, ao
+
+
+def _case(n_ctx, hq, hkv, n_stripes, seed, **kw):
+    from anchor_attn.synthetic import make_qkv
+    q, k, v, pos = make_qkv(n_ctx, hq, hkv, n_stripes=n_stripes, seed=seed, **kw)
+    return q, k, v, pos
+
+
+@pytest.fixture(scope="module")
+def llama_small(mods):
+    """3 big blocks, GQA 4:1 (Llama grouping), 96 stripes."""
+    _, _, _, ao = mods
+    q, k, v, pos = _case(3 * S, 8, 2, 96, seed=21)
+    Q, K, V = _np(q, k, v)
+    res = ao.anchor_attn_reference(Q, K, V, difference=12.0)
+    return (q.cuda(), k.cuda(), v.cuda()), (Q, K, V), res
+
+
+def _packed_lists(hip, coords, counts, N):
+    coords = coords.cpu().numpy()
+    counts = counts.cpu().numpy().reshape(coords.shape[0], coords.shape[1], -1)
+    lib = hip.lib()
+    out = []
+    for b in range(coords.shape[0]):
+        pb = []
+        for h in range(coords.shape[1]):
+            ph = []
+            for bb in range(counts.shape[2]):
+                off = lib.aa_coords_offset(bb, BS, STEP)
+                ph.append(coords[b, h, off:off + counts[b, h, bb]].copy())
+            pb.append(ph)
+        out.append(pb)
+    return out, counts
+
+
+def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused):
+    """Sets equal except excused keys (flip distance < BAND); returns number of excused keys."""
+    B, Hq = got_counts.shape[:2]
+    group = Hq // K.shape[1]
+    excused = 0
+    for b in range(B):
+        for h in range(Hq):
+            qbar = abar = mean = None
+            for bb in range(got_counts.shape[2]):
+                g, w = got[b][h][bb], want[b][h][bb]
+                assert np.all(np.diff(g) > 0), "index list must be strictly ascending"
+                if g.size:
+                    assert g[0] >= BS and g[-1] < bb * S - BS
+                sym = np.setxor1d(g, w)
+                if sym.size == 0:
+                    continue
+                if qbar is None:
+                    qbar = ao.pooled_queries(Q[b, h], BS)
+                    abar, mean = ao.pooled_anchors(M[b, h], BS)
+                rows = slice(bb * STEP, (bb + 1) * STEP)
+                for j in sym:
+                    d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta)
+                    assert d < BAND, f"key {j} (b={b},h={h},bb={bb}) differs and is {d:.4g} from any decision flip"
+                    excused += 1
+    assert excused <= max_excused, f"{excused} near-threshold disagreements"
+    return excused
+
+
+# ------------------------------------------------------------------------------------ stage 1
+def test_stage1_anchor_matches_oracle(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, B, H, N, D, SM)
+    torch.cuda.synchronize()
+    M, L, A = M.cpu().numpy(), L.cpu().numpy(), st.acc_rows(Acc).cpu().numpy()
+    assert np.isfinite(M).all() and np.isfinite(L).all() and np.isfinite(A).all()
+    np.testing.assert_allclose(M, res.M, atol=3e-4)
+    np.testing.assert_allclose(L, res.L, rtol=5e-4)
+    err = np.abs(A / L[..., None] - res.Acc / res.L[..., None])
+    assert err.max() < 6e-3 and err.mean() < 3e-4
+
+
+def test_stage1_fp32_scale_switch(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(q[:, :2], k[:, :1], v[:, :1], 1, 1, BS, STEP, B, 2, N, D, SM, scale_mode=hip.AA_SCALE_FP32)
+    M2, _, _ = ao.stage1_anchor(Q[:, :2], K[:, :1], V[:, :1], SM, scale_mode="fp32")
+    np.testing.assert_allclose(M.cpu().numpy(), M2, atol=3e-4)
+    assert np.abs(M2 - res.M[:, :2]).max() > 1e-2  # the two chains are measurably different
+
+
+# ------------------------------------------------------------------------------------ stage 2
+def test_pooling_is_bit_exact(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    Mdev = torch.from_numpy(res.M).cuda()
+    qbar, abar = st.pool_q_anchor(q, Mdev, BS)
+    qbar, abar = _np(qbar, abar)
+    for h in range(q.shape[1]):
+        assert np.array_equal(qbar[0, h], ao.pooled_queries(Q[0, h], BS))
+        assert np.array_equal(abar[0, h], ao.pooled_anchors(res.M[0, h], BS)[0])
+
+
+@pytest.mark.parametrize("theta", [12.0, 14.0, 9.0])
+def test_stage2_select_matches_oracle_given_same_anchors(mods, llama_small, theta):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    B, H, N, _ = q.shape
+    Mdev = torch.from_numpy(res.M).cuda()
+    coords, counts = st.select_stripes_packed(q, k, Mdev, BS, STEP, theta * LOG2E, B, H, N, D, SM)
+    got, got_counts = _packed_lists(hip, coords, counts, N)
+    want, want_counts = ao.stage2_select(Q, K, res.M, SM, theta)
+    _assert_index_parity(ao, got, got_counts, want, Q, K, res.M, theta, max_excused=4)
+    assert got_counts[:, :, 0].sum() == 0
+
+
+def test_stage2_closed_forms_on_gpu(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    B, H, N, _ = q.shape
+    Mdev = torch.from_numpy(res.M).cuda()
+    coords, counts = st.select_stripes_packed(q, k, Mdev, BS, STEP, 1e4, B, H, N, D, SM)
+    got, got_counts = _packed_lists(hip, coords, counts, N)
+    for h in range(H):
+        for bb in range(N // S):
+            want = np.arange(BS, bb * S - BS, dtype=np.int32) if bb else np.zeros(0, np.int32)
+            assert np.array_equal(got[0][h][bb], want)
+    _, counts = st.select_stripes_packed(q, k, Mdev, BS, STEP, -1e4, B, H, N, D, SM)
+    assert int(counts.sum()) == 0
+    # reference-layout view
+    tc, cnt = st.anchor_attn_step_2(q.contiguous(), k.repeat_interleave(H // k.shape[1], dim=1).contiguous(), Mdev, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM)
+    assert tc.shape == (B, H, N // S, N) and cnt.shape == (B, H, N // S, 1)
+    assert np.array_equal(tc.cpu().numpy(), ao.coords_to_reference_layout(res.coords, res.counts, N))
+
+
+# ------------------------------------------------------------------------------------ stage 3
+def test_stage3_matches_oracle_given_same_state(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), (Q, K, V), res = llama_small
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(q, k, M, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM)
+    out = v4._stage3(q, k, v, coords, counts, L, M, Acc, SM, BS, STEP)
+    torch.cuda.synchronize()
+    got_lists, got_counts = _packed_lists(hip, coords, counts, N)
+    want = ao.stage3_sparse(Q, K, V, got_lists, got_counts, M.cpu().numpy(), L.cpu().numpy(),
+                            st.acc_rows(Acc).cpu().numpy(), SM)
+    err = np.abs(out.float().cpu().numpy() - want)
+    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+
+
+# ------------------------------------------------------------------------------------ whole operator
+def _end_to_end(mods, q, k, v, theta, max_excused=6, rope_note=""):
+    hip, v4, st, ao = mods
+    Q, K, V = _np(q, k, v)
+    res = ao.anchor_attn_reference(Q, K, V, difference=theta)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out, ratio = v4.anchor_attn(qd, kd, vd, difference=theta)
+    B, H, N, _ = q.shape
+    # stage outputs for index parity come from the staged entry points on the same inputs
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, theta * LOG2E, B, H, N, D, SM)
+    got, got_counts = _packed_lists(hip, coords, counts, N)
+    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused)
+    err = np.abs(out.float().cpu().numpy() - res.out)
+    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
+    want_ratio = got_counts.sum() / ((B * H * N * N / (BS * STEP)) // 2)
+    assert abs(float(ratio) - want_ratio) < 1e-6
+    return res, out
+
+
+def test_anchor_attn_end_to_end_llama_grouping(mods, llama_small):
+    (q, k, v), _, _ = llama_small
+    res, out = _end_to_end(mods, q.cpu(), k.cpu(), v.cpu(), 12.0)
+    assert res.counts.sum() > 0
+
+
+def test_anchor_attn_end_to_end_qwen_grouping(mods):
+    """GQA 7:1 (not a power of two), RoPE base 1e6, 4 big blocks."""
+    q, k, v, _ = _case(4 * S, 7, 1, 128, seed=33, rope_base=1e6)
+    _end_to_end(mods, q, k, v, 12.0)
+
+
+def test_anchor_attn_config0_shape(mods):
+    """BASELINE config 0 shape (32/8 heads, N=4096, 64 stripes): every candidate lies inside the
+    init window, so selected keys are all double-counted."""
+    q, k, v, _ = _case(2 * S, 32, 8, 64, seed=0)
+    res, _ = _end_to_end(mods, q, k, v, 12.0)
+    assert res.counts.sum() > 0
+
+
+def test_anchor_attn_dense_regime_literal_qbar(mods):
+    """literal qbar: every candidate is selected (ratio ~ 1), stage 3 walks full index lists."""
+    q, k, v, _ = _case(3 * S, 2, 1, 32, seed=4, qbar_mode="literal")
+    res, _ = _end_to_end(mods, q, k, v, 12.0, max_excused=50)
+    assert res.counts[0, 0, 2] > 3000
+
+
+def test_theta_minus_inf_two_big_blocks_equals_library_attention(mods):
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(2 * S, 4, 2, 32, seed=5)
+    out, ratio = v4.anchor_attn(q.cuda(), k.cuda(), v.cuda(), difference=-1e4)
+    assert float(ratio) == 0.0
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    err = (out.cpu().double() - ref).abs()
+    assert err.max() < 3e-2 and err.mean() < 2e-3
+
+
+def test_dense_baseline_equals_library_attention(mods):
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(3 * S, 4, 2, 32, seed=6)
+    out = v4.dense_causal_attention(q.cuda(), k.cuda(), v.cuda())
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    err = (out.cpu().double() - ref).abs()
+    assert err.max() < 2e-2 and err.mean() < 1e-3
+
+
+def test_strided_and_repeated_inputs_give_identical_results(mods, llama_small):
+    """[B,N,H,D] storage (HF layout) and pre-repeated K/V must give bit-identical outputs."""
+    hip, v4, st, ao = mods
+    (q, k, v), _, _ = llama_small
+    base = v4.anchor_attn(q, k, v, return_computational_ratio=False)
+    qs = q.transpose(1, 2).contiguous().transpose(1, 2)
+    ks = k.transpose(1, 2).contiguous().transpose(1, 2)
+    vs = v.transpose(1, 2).contiguous().transpose(1, 2)
+    assert not qs.is_contiguous()
+    o_buf = torch.empty_like(q.transpose(1, 2)).transpose(1, 2)
+    o2 = v4.anchor_attn(qs, ks, vs, return_computational_ratio=False, out=o_buf)
+    assert o2.data_ptr() == o_buf.data_ptr() and torch.equal(o2, base)
+    g = q.shape[1] // k.shape[1]
+    o3 = v4.anchor_attn(q, k.repeat_interleave(g, 1), v.repeat_interleave(g, 1), return_computational_ratio=False)
+    assert torch.equal(o3, base)
+
+
+def test_repeatable_bit_for_bit(mods, llama_small):
+    hip, v4, st, ao = mods
+    (q, k, v), _, _ = llama_small
+    B, H, N, _ = q.shape
+    a = v4.anchor_attn_test_time(q, k, v)
+    b = v4.anchor_attn_test_time(q, k, v)
+    assert torch.equal(a[0], b[0]) and float(a[1]) == float(b[1])
+    assert len(a) == 4 and a[2] > 0 and a[3] > 0
+    assert len(v4.anchor_attn_test_time(q, k, v, return_computational_ratio=False)) == 3
+    c, r = v4.anchor_attn_without_anchor(q, k, v)
+    assert torch.equal(c, a[0])
+
+
+def test_entry_assertions_and_error_codes(mods):
+    hip, v4, st, ao = mods
+    q = torch.zeros(1, 2, 2048, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(AssertionError):
+        v4.anchor_attn(q, q, q, step=8)
+    with pytest.raises(AssertionError):
+        v4.anchor_attn(q[:, :, :1024], q[:, :, :1024], q[:, :, :1024])
+    with pytest.raises(AssertionError):
+        v4.anchor_attn(q.float(), q.float(), q.float())
+    with pytest.raises(hip.AnchorAttnHipError):
+        v4.anchor_attn(q, q, q, block_size=64, step=32)  # block_size 64 is not built
+    lib = hip.lib()
+    rc = lib.aa_dense_causal_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 2, 2048, 128, 0.1, None)
+    assert rc == 1 and b"NULL" in lib.aa_last_error()
+
+
+# ------------------------------------------------------------------------------------ larger sizes
+def test_constant_values_at_32k(mods):
+    """Size-independent property at the 32k shape: if every V row is the same vector, every output
+    row equals it, whatever was selected (checks normalisation across all three stages)."""
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(16 * S, 8, 2, 512, seed=7)
+    row = torch.linspace(-2, 2, D).to(torch.bfloat16)
+    vc = row.expand_as(v).contiguous()
+    out, ratio = v4.anchor_attn(q.cuda(), k.cuda(), vc.cuda())
+    assert 0 < float(ratio) < 0.2
+    err = (out.float().cpu() - row.float()).abs()
+    assert err.max() <= 2e-2
