@@ -51,6 +51,10 @@ int check_dims(const Dims& d, const char* who) {
     set_error("%s: n_ctx %d is not a multiple of block_size*step = %d", who, d.n_ctx, d.block_size * d.step);
     return AA_EUNSUPPORTED;
   }
+  if (d.n_ctx > (1 << 20)) {
+    set_error("%s: n_ctx %d is larger than 1048576", who, d.n_ctx);
+    return AA_EUNSUPPORTED;
+  }
   if ((int64_t)d.batch * d.n_q_heads * (d.n_ctx / 128) > 0x7fffffffLL) {
     set_error("%s: problem too large for one launch", who);
     return AA_EUNSUPPORTED;
@@ -70,6 +74,10 @@ int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, const char
   if (sn < 128) {
     set_error("%s: %s row stride %lld is smaller than head_dim", who, name, (long long)sn);
     return AA_EBADARG;
+  }
+  if (sn > (int64_t)1 << 14) {  // the kernels address rows of one head with 32-bit byte offsets
+    set_error("%s: %s row stride %lld is larger than 16384 elements", who, name, (long long)sn);
+    return AA_EUNSUPPORTED;
   }
   return AA_OK;
 }

@@ -8,43 +8,47 @@
 // so that in the 32x32 accumulator layout a lane holds one query column: the soft-max statistics
 // of a query are then plain per-lane scalars (one exchange with the lane 32 positions away
 // completes the row max).  The second product is computed transposed as well,
-//   O^T[d][query] += V^T[d][key] . P^T[key][query]  (A = V^T from LDS, B = P^T straight from the
-// S^T accumulator registers, rounded to bf16) - P never travels through LDS.
-// The contraction slot k = 8*(lane/32) + e of MFMA step s of key block kb is fed from accumulator
-// register 8*s + e, i.e. key 32*kb + 16*s + 8*(e/4) + 4*(lane/32) + e%4.  V^T is therefore
-// written to LDS with bits 2 and 3 of the key index swapped ("slot" order), which makes every
-// lane's eight V^T operands one contiguous 16-byte LDS read.
+//   O^T[d][query] += V^T[d][key] . P^T[key][query]  (A = V^T, B = P^T straight from the S^T
+// accumulator registers, rounded to bf16) - P never travels through LDS.
+// The contraction slot k = 8*(lane/32) + e of MFMA step st of key block kb is fed from accumulator
+// register 8*st + e, i.e. key 32*kb + 16*st + 8*(e/4) + 4*(lane/32) + e%4: two runs of four
+// consecutive keys.  V sits row-major in LDS exactly as it is in memory, and each run of four keys
+// at one head-dim column is fetched with the transposing LDS read ds_read_b64_tr_b16 (within a group
+// of 16 lanes, lane i receives column i of the 4x16 block whose rows the group's lanes point at).
 //
 // Work-group = 4 waves = 128*QB query rows; keys are consumed 64 at a time through a
-// double-buffered LDS tile (K row-major, padded to 272-byte rows; V^T padded to 144-byte rows, both
-// conflict-free for 16-byte reads by 8 consecutive lanes).
+// double-buffered LDS tile (K and V rows padded to 272 bytes).
 #include "aa_common.h"
 #include "aa_kernels.h"
 
 namespace aa {
 
-constexpr int kBN = 64;          // keys per LDS tile
-constexpr int kKsStride = 136;   // bf16 per K row in LDS
-constexpr int kVtStride = 72;    // bf16 per V^T row in LDS
+constexpr int kBN = 64;        // keys per LDS tile
+constexpr int kRowStride = 136;  // bf16 per K/V row in LDS (256 B of data + 16 B pad)
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
+
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
 
 template <int QB>
 struct FlashSmem {
   union {
     struct {
-      __bf16 ks[2][kBN * kKsStride];
-      __bf16 vt[2][128 * kVtStride];
+      __bf16 k[2][kBN * kRowStride];
+      __bf16 v[2][kBN * kRowStride];
     } t;
     __bf16 os[4][32 * QB * kOsStride];  // epilogue staging, reuses the tile space
   };
 };
 
-__device__ __forceinline__ void scale_q8(const uint4& raw, float sm_scale, int scale_mode, bf16x8& dst) {
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+__device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale, const bool bf16_chain) {
+  const uint32_t w[4] = {raw[0], raw[1], raw[2], raw[3]};
   uint32_t o[4];
-  if (scale_mode == 0) {  // bf16 chain: bf16(bf16(q * bf16(sm_scale)) * bf16(log2e))
+  if (bf16_chain) {  // bf16(bf16(q * bf16(sm_scale)) * bf16(log2e))
     const float s16 = rn16(sm_scale), c16 = rn16(kLog2e);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -55,12 +59,50 @@ __device__ __forceinline__ void scale_q8(const uint4& raw, float sm_scale, int s
 #pragma unroll
     for (int i = 0; i < 4; ++i) o[i] = pack_bf16((bf16_lo(w[i]) * sm_scale) * kLog2e, (bf16_hi(w[i]) * sm_scale) * kLog2e);
   }
-  uint4 packed = {o[0], o[1], o[2], o[3]};
-  dst = *reinterpret_cast<bf16x8*>(&packed);
+  const u32x4 packed = {o[0], o[1], o[2], o[3]};
+  return *reinterpret_cast<const bf16x8*>(&packed);
+}
+
+// Registers that carry one K/V tile from global memory to LDS.
+struct TileRegs {
+  u32x4 k[4];
+  u32x4 v[4];
+};
+
+// Thread t moves 16-byte chunk (t & 15) of tile rows (t >> 4) + 16*j, j = 0..3, for K and for V.
+// `kb`/`vb` are the wave-uniform head bases; row offsets are 32-bit byte offsets.
+template <int MODE>
+__device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const char* vb, const uint32_t k_row_bytes,
+                                          const uint32_t v_row_bytes, const int key0, const int tid, const int32_t* cbase,
+                                          const int cnt) {
+  const int row0 = tid >> 4;
+  const uint32_t col = (tid & 15) * 16;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = row0 + 16 * j;
+    uint32_t key;
+    if (MODE == kSparse) {
+      key = (key0 + row < cnt) ? (uint32_t)cbase[key0 + row] : 0u;  // tail lanes read row 0, masked later
+    } else {
+      key = (uint32_t)(key0 + row);
+    }
+    r.k[j] = *reinterpret_cast<const u32x4*>(kb + (key * k_row_bytes + col));
+    r.v[j] = *reinterpret_cast<const u32x4*>(vb + (key * v_row_bytes + col));
+  }
+}
+
+__device__ __forceinline__ void tile_store(const TileRegs& r, __bf16* ks, __bf16* vs, const int tid) {
+  const int row0 = tid >> 4, c = tid & 15;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int off = (row0 + 16 * j) * kRowStride + 8 * c;
+    *reinterpret_cast<u32x4*>(ks + off) = r.k[j];
+    *reinterpret_cast<u32x4*>(vs + off) = r.v[j];
+  }
 }
 
 template <int QB, int MODE>
-__global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
+__global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const FlashArgs p) {
   __shared__ __attribute__((aligned(16))) FlashSmem<QB> sm;
   constexpr int BM = 128 * QB;
 
@@ -87,18 +129,38 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 
   const __bf16* qp = p.q + b * p.q_sb + hq * p.q_sh;
-  const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
-  const __bf16* vp = p.v + b * p.v_sb + kvh * p.v_sh;
+  const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
+  const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
+  const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
+
+  // ---- tile schedule -------------------------------------------------------------------------
+  int n_tiles, n_init = 0, cnt = 0;
+  const int32_t* cbase = nullptr;
+  if (MODE == kAnchor) {
+    n_init = min(S, R0 + BM) / kBN;
+    n_tiles = n_init + (bb >= 1 ? (R0 + BM - bb * S) / kBN : 0);
+  } else if (MODE == kDense) {
+    n_tiles = (R0 + BM) / kBN;
+  } else {
+    cnt = p.counts[bh * (p.n_ctx / S) + bb];
+    cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
+    n_tiles = (cnt + kBN - 1) / kBN;
+  }
+  // first key (anchor, dense) or first list position (sparse) of tile i
+#define AA_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
+
+  TileRegs tr;
+  if (n_tiles > 0) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(0), tid, cbase, cnt);
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
   bf16x8 qreg[QB][8];
+  {
+    const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    const __bf16* row = qp + (int64_t)(wr0 + 32 * qb + c32) * p.q_sn + 8 * half;
+    for (int qb = 0; qb < QB; ++qb) {
+      const __bf16* row = qp + (int64_t)(wr0 + 32 * qb + c32) * p.q_sn + 8 * half;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const uint4 raw = *reinterpret_cast<const uint4*>(row + 16 * ks);
-      scale_q8(raw, p.sm_scale, MODE == kAnchor ? p.scale_mode : 1, qreg[qb][ks]);
+      for (int ks = 0; ks < 8; ++ks) qreg[qb][ks] = scale_q8(*reinterpret_cast<const u32x4*>(row + 16 * ks), p.sm_scale, chain);
     }
   }
 
@@ -110,7 +172,7 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
     for (int qb = 0; qb < QB; ++qb) {
       const int row = wr0 + 32 * qb + c32;
       m_run[qb] = p.M[bh * p.n_ctx + row];
-      l_run[qb] = half == 0 ? p.L[bh * p.n_ctx + row] : 0.f;  // halves are summed at the end
+      l_run[qb] = half == 0 ? p.L[bh * p.n_ctx + row] : 0.f;  // the two halves are summed at the end
       const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + row / 32) * 16) * 256 + lane * 4;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
@@ -133,103 +195,39 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
     }
   }
 
-  // ---- tile schedule -------------------------------------------------------------------------
-  int n_tiles, n_init = 0, cnt = 0;
-  const int32_t* cbase = nullptr;
-  if (MODE == kAnchor) {
-    n_init = min(S, R0 + BM) / kBN;
-    n_tiles = n_init + (bb >= 1 ? (R0 + BM - bb * S) / kBN : 0);
-  } else if (MODE == kDense) {
-    n_tiles = (R0 + BM) / kBN;
-  } else {
-    cnt = p.counts[bh * (p.n_ctx / S) + bb];
-    cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
-    n_tiles = (cnt + kBN - 1) / kBN;
-  }
-  auto tile_key0 = [&](int i) -> int {
-    if (MODE == kAnchor) return i < n_init ? i * kBN : bb * S + (i - n_init) * kBN;
-    return i * kBN;  // dense: key index; sparse: position in the index list
-  };
-
-  uint4 kreg[4];
-  uint32_t vreg[4][4];
-  auto issue_loads = [&](int i) {
-    const int key0 = tile_key0(i);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int id = tid + 256 * j, row = id >> 4, c = id & 15;
-      int64_t key = key0 + row;
-      if (MODE == kSparse) key = (key0 + row < cnt) ? cbase[key0 + row] : 0;
-      kreg[j] = *reinterpret_cast<const uint4*>(kp + key * p.k_sn + 8 * c);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int g4 = 4 * (wave + 4 * j);  // first of the four keys this wave transposes
-      int64_t keys[4];
-      if (MODE == kSparse) {
-        const int4 ids = *reinterpret_cast<const int4*>(cbase + key0 + g4);
-        keys[0] = key0 + g4 + 0 < cnt ? ids.x : 0;
-        keys[1] = key0 + g4 + 1 < cnt ? ids.y : 0;
-        keys[2] = key0 + g4 + 2 < cnt ? ids.z : 0;
-        keys[3] = key0 + g4 + 3 < cnt ? ids.w : 0;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) keys[e] = key0 + g4 + e;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) vreg[j][e] = *reinterpret_cast<const uint32_t*>(vp + keys[e] * p.v_sn + 2 * lane);
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int id = tid + 256 * j, row = id >> 4, c = id & 15;
-      *reinterpret_cast<uint4*>(&sm.t.ks[buf][row * kKsStride + 8 * c]) = kreg[j];
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int gq = wave + 4 * j;                                        // key group (4 keys)
-      const int slot0 = 4 * ((gq & ~3) | ((gq & 1) << 1) | ((gq >> 1) & 1));  // bits 2,3 of the key swapped
-      const uint32_t* d = vreg[j];
-      uint2 lo, hi;
-      lo.x = (d[0] & 0xffffu) | (d[1] << 16);
-      lo.y = (d[2] & 0xffffu) | (d[3] << 16);
-      hi.x = (d[0] >> 16) | (d[1] & 0xffff0000u);
-      hi.y = (d[2] >> 16) | (d[3] & 0xffff0000u);
-      *reinterpret_cast<uint2*>(&sm.t.vt[buf][(2 * lane) * kVtStride + slot0]) = lo;
-      *reinterpret_cast<uint2*>(&sm.t.vt[buf][(2 * lane + 1) * kVtStride + slot0]) = hi;
-    }
-  };
-
-  if (n_tiles > 0) {
-    issue_loads(0);
-    store_tile(0);
-  }
+  if (n_tiles > 0) tile_store(tr, sm.t.k[0], sm.t.v[0], tid);
   __syncthreads();
+
+  // per-lane LDS offsets (in bf16 elements)
+  const int k_rd = c32 * kRowStride + 8 * half;  // K row c32 (+32*kb), columns 8*half (+16*ks)
+  // transposing V read: group of 16 lanes covers 16 head-dim columns, lane i points at row i/4, 4 columns from 4*(i%4)
+  const int v_rd = (4 * half + ((lane & 15) >> 2)) * kRowStride + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   for (int i = 0; i < n_tiles; ++i) {
     const int buf = i & 1;
-    const int key0 = tile_key0(i);
-    if (i + 1 < n_tiles) issue_loads(i + 1);
+    const int key0 = AA_TILE_KEY0(i);
+    if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
 
     // a wave whose rows all lie above this tile (causal) has nothing to do
     const bool wave_active = (MODE == kSparse) || (key0 <= wr0 + 32 * QB - 1);
     if (wave_active) {
+      const __bf16* ks_ = sm.t.k[buf] + k_rd;
       // ---- S^T = K Q^T ------------------------------------------------------------------------
       floatx16 s[2][QB];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[kb][qb][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(&sm.t.ks[buf][(32 * kb + c32) * kKsStride + 16 * ks + 8 * half]);
+          const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * ks);
 #pragma unroll
-          for (int qb = 0; qb < QB; ++qb) s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[qb][ks], s[kb][qb], 0, 0, 0);
+          for (int qb = 0; qb < QB; ++qb) {
+            if (ks == 0) {
+              const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[qb][ks], zero, 0, 0, 0);
+            } else {
+              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[qb][ks], s[kb][qb], 0, 0, 0);
+            }
+          }
         }
 
       // ---- masks ------------------------------------------------------------------------------
@@ -284,11 +282,11 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
           }
 #pragma unroll
           for (int st = 0; st < 2; ++st) {
-            uint4 w;
-            w.x = pack_bf16(pv[8 * st + 0], pv[8 * st + 1]);
-            w.y = pack_bf16(pv[8 * st + 2], pv[8 * st + 3]);
-            w.z = pack_bf16(pv[8 * st + 4], pv[8 * st + 5]);
-            w.w = pack_bf16(pv[8 * st + 6], pv[8 * st + 7]);
+            u32x4 w;
+            w[0] = pack_bf16(pv[8 * st + 0], pv[8 * st + 1]);
+            w[1] = pack_bf16(pv[8 * st + 2], pv[8 * st + 3]);
+            w[2] = pack_bf16(pv[8 * st + 4], pv[8 * st + 5]);
+            w[3] = pack_bf16(pv[8 * st + 6], pv[8 * st + 7]);
             pfrag[kb][qb][st] = *reinterpret_cast<bf16x8*>(&w);
           }
         }
@@ -305,21 +303,28 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
       }
 
       // ---- O^T += V^T P^T ---------------------------------------------------------------------
+      const __bf16* vs_ = sm.t.v[buf] + v_rd;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
           for (int db = 0; db < 4; ++db) {
-            const bf16x8 a = *reinterpret_cast<const bf16x8*>(&sm.t.vt[buf][(32 * db + c32) * kVtStride + 32 * kb + 16 * st + 8 * half]);
+            const __bf16* src = vs_ + (32 * kb + 16 * st) * kRowStride + 32 * db;
+            const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(src));
+            const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(src + 8 * kRowStride));
+            typedef short shortx8 __attribute__((ext_vector_type(8)));
+            const shortx8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            const bf16x8 a = *reinterpret_cast<const bf16x8*>(&av);
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) acc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[kb][qb][st], acc[db][qb], 0, 0, 0);
           }
     }
 
-    if (i + 1 < n_tiles) store_tile(buf ^ 1);
+    if (i + 1 < n_tiles) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
     __syncthreads();
   }
+#undef AA_TILE_KEY0
 
   // ---- epilogue --------------------------------------------------------------------------------
   if (MODE == kAnchor) {
@@ -353,10 +358,10 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
-          uint2 w;
-          w.x = pack_bf16(acc[db][qb][rg * 4 + 0] * inv, acc[db][qb][rg * 4 + 1] * inv);
-          w.y = pack_bf16(acc[db][qb][rg * 4 + 2] * inv, acc[db][qb][rg * 4 + 3] * inv);
-          *reinterpret_cast<uint2*>(&os[(32 * qb + c32) * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
+          u32x2 w;
+          w[0] = pack_bf16(acc[db][qb][rg * 4 + 0] * inv, acc[db][qb][rg * 4 + 1] * inv);
+          w[1] = pack_bf16(acc[db][qb][rg * 4 + 2] * inv, acc[db][qb][rg * 4 + 3] * inv);
+          *reinterpret_cast<u32x2*>(&os[(32 * qb + c32) * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
         }
     }
     __syncthreads();
@@ -364,8 +369,8 @@ __global__ void __launch_bounds__(256) flash_kernel(const FlashArgs p) {
 #pragma unroll
     for (int it = 0; it < 8 * QB; ++it) {
       const int r = it * 4 + (lane >> 4), c = lane & 15;
-      const uint4 w = *reinterpret_cast<const uint4*>(&os[r * kOsStride + 8 * c]);
-      *reinterpret_cast<uint4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c) = w;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(&os[r * kOsStride + 8 * c]);
+      *reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c) = w;
     }
   }
 }

@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the AnchorAttention prefill operator on one MI355X.
+
+A step is one full operator call (stage 1 -> pooling -> stage 2 -> stage 3) for one attention layer
+on seeded synthetic q/k/v already resident in HBM.  The default workload is the headline one:
+Llama-3.1-8B layer shape (32 q heads / 8 KV heads, head_dim 128) at 131072 tokens, theta 12.
+Prints ONE JSON line.  `value` is effective TFLOP/s = (F1 + F2 + F3) / time with
+  F1 = Hq * T1 * 4*128*128*D,  T1 = 136 + (nBB-1)*392 useful 128x128 tiles of the anchor window pass,
+  F2 = Hq * 2*16*D * sum_bb max(bb*S - 256, 0)   (pooled-query x candidate-key scores),
+  F3 = 4*D*S * sum(counts)                        (selected keys x the 2048 queries of a big block).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "anchor-attention_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (n_ctx, hq, hkv, rope_base, n_stripes, stripe_dist)
+    "config0_llama8b_4k": (4096, 32, 8, 5e5, 64, "uniform"),
+    "config1_llama8b_32k": (32768, 32, 8, 5e5, 512, "uniform"),
+    "config2_llama8b_128k": (131072, 32, 8, 5e5, 655, "powerlaw"),
+    "config3_qwen7b_64k": (65536, 28, 4, 1e6, 328, "uniform"),
+}
+
+
+def flops(hq, n_ctx, sum_counts, D=128, S=2048):
+    n_bb = n_ctx // S
+    t1 = 136 + (n_bb - 1) * 392
+    f1 = hq * t1 * 4 * 128 * 128 * D
+    f2 = hq * 2 * 16 * D * sum(max(bb * S - 256, 0) for bb in range(n_bb))
+    f3 = 4 * D * S * sum_counts
+    return f1, f2, f3
+
+
+def make_inputs(name, seed, qbar_mode, device):
+    """Same construction as anchor_attn.synthetic.make_qkv, but drawn on the GPU (a 128k-token layer
+    is 0.5 G random numbers per tensor); stripe positions still come from the CPU generator."""
+    import torch
+    from anchor_attn.synthetic import stripe_positions
+    n_ctx, hq, hkv, base, n_stripes, dist = WORKLOADS[name]
+    D = 128
+    g = torch.Generator(device=device).manual_seed(seed)
+    cg = torch.Generator(device="cpu").manual_seed(seed)
+    inv = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float64, device=device) / D))
+    ang = torch.arange(n_ctx, dtype=torch.float64, device=device)[:, None] * inv[None, :]
+    cos = torch.cat([ang.cos(), ang.cos()], -1).float()
+    sin = torch.cat([ang.sin(), ang.sin()], -1).float()
+    del ang
+
+    def rope(x):
+        x1, x2 = x[..., : D // 2], x[..., D // 2:]
+        return x * cos + torch.cat([-x2, x1], -1) * sin
+
+    group = hq // hkv
+    pos = stripe_positions(n_ctx, n_stripes, dist, cg).to(device)
+    u = torch.randn(hkv, D, generator=cg).to(device)
+    qbar = u / u.norm(dim=-1, keepdim=True) * math.sqrt(16.0 / (4.0 / math.sqrt(D)))
+    q = torch.empty(1, hq, n_ctx, D, dtype=torch.bfloat16, device=device)
+    k = torch.empty(1, hkv, n_ctx, D, dtype=torch.bfloat16, device=device)
+    v = torch.randn(1, hkv, n_ctx, D, generator=g, device=device).to(torch.bfloat16)
+    qsum = torch.zeros(hkv, D, device=device)
+    kf = []
+    for h in range(hkv):
+        kf.append(rope(torch.randn(n_ctx, D, generator=g, device=device)))
+    for h in range(hq):
+        x = rope(torch.randn(n_ctx, D, generator=g, device=device))
+        if qbar_mode == "shared":
+            x = x + qbar[h // group]
+        else:
+            qsum[h // group] += x.mean(0) / group
+        q[0, h] = x.to(torch.bfloat16)
+    if qbar_mode != "shared":
+        qbar = qsum
+    for h in range(hkv):
+        x = kf[h]
+        x[0] += 4.0 * qbar[h]
+        x[pos] += 2.0 * qbar[h]
+        k[0, h] = x.to(torch.bfloat16)
+    return q, k, v
+
+
+def cpu_baseline():
+    """The CPU oracle (our numpy restatement of the reference algorithm - the reference has no CPU
+    path of its own) timed on this host on a bounded sample: the config-0 shape (N=4096, 32/8 heads)."""
+    import numpy as np
+    from anchor_attn.synthetic import make_qkv
+    from oracle import anchor_oracle as ao
+    n_ctx, hq, hkv = 4096, 32, 8
+    q, k, v, _ = make_qkv(n_ctx, hq, hkv, n_stripes=64, seed=0)
+    Q, K, V = (t.float().numpy() for t in (q, k, v))
+    t0 = time.time()
+    res = ao.anchor_attn_reference(Q, K, V, difference=12.0)
+    dt = time.time() - t0
+    f1, f2, f3 = flops(hq, n_ctx, int(res.counts.sum()))
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {
+        "value": (f1 + f2 + f3) / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"numpy oracle, one layer at N={n_ctx}, {hq}q/{hkv}kv heads, theta=12, {dt * 1e3:.0f} ms "
+                  f"(BLAS threads={cores})",
+        "ms": dt * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="config2_llama8b_128k", choices=sorted(WORKLOADS))
+    ap.add_argument("--theta", type=float, default=12.0)
+    ap.add_argument("--qbar-mode", default="shared", choices=["shared", "literal"])
+    ap.add_argument("--seed", type=int, default=2024)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the operator is embarrassingly parallel over KV-head "
+                 "groups; see DESIGN.md for how it would shard) - run with --gpus 1")
+
+    import torch
+    from anchor_attn.src.ops import _hip, anchor_attn_v4 as v4, anchor_step_1_2_v2 as st
+    _hip.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    n_ctx, hq, hkv, _, _, _ = WORKLOADS[args.workload]
+    D, BS, STEP, S = 128, 128, 16, 2048
+    sm = 1.0 / math.sqrt(D)
+    q, k, v = make_inputs(args.workload, args.seed, args.qbar_mode, dev)
+    out = torch.empty_like(q)
+    torch.cuda.synchronize()
+
+    # ---- timed region: K calls of the public operator -----------------------------------------
+    for _ in range(args.warmup):
+        v4.anchor_attn(q, k, v, difference=args.theta, return_computational_ratio=False, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        v4.anchor_attn(q, k, v, difference=args.theta, return_computational_ratio=False, out=out)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- same kernels, staged, with events between them on the launch stream -------------------
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    theta2 = args.theta * v4.LOG2E
+    counts = None
+    for i in range(args.steps):
+        ev[i][0].record()
+        L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, 1, hq, n_ctx, D, sm)
+        ev[i][1].record()
+        qbar, abar = st.pool_q_anchor(q, M, BS)
+        ev[i][2].record()
+        lib = _hip.lib()
+        if counts is None:
+            mask = torch.empty((lib.aa_mask_words(1, hq, n_ctx, BS, STEP),), dtype=torch.int32, device=dev)
+            coords = torch.empty((1, hq, lib.aa_coords_entries_per_head(n_ctx, BS, STEP)), dtype=torch.int32, device=dev)
+            counts = torch.empty((1, hq, n_ctx // S, 1), dtype=torch.int32, device=dev)
+        _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(k), mask.data_ptr(), coords.data_ptr(),
+                                        counts.data_ptr(), 1, hq, hkv, n_ctx, D, BS, STEP, sm, theta2,
+                                        torch.cuda.current_stream().cuda_stream))
+        ev[i][3].record()
+        v4._stage3(q, k, v, coords, counts, L, M, Acc, sm, BS, STEP, out=out)
+        ev[i][4].record()
+        del L, M, Acc
+    torch.cuda.synchronize()
+    st_ms = [sum(ev[i][j].elapsed_time(ev[i][j + 1]) for i in range(args.steps)) / args.steps for j in range(4)]
+    sum_counts = int(counts.sum())
+    f1, f2, f3 = flops(hq, n_ctx, sum_counts)
+    ratio = sum_counts / ((1 * hq * n_ctx * n_ctx / (BS * STEP)) // 2)
+    dense_flops = 4 * D * hq * n_ctx * (n_ctx + 1) / 2
+
+    stage_tflops = [f1 / st_ms[0] / 1e9, None, f2 / st_ms[2] / 1e9, f3 / st_ms[3] / 1e9 if f3 else 0.0]
+    # the dominant kernel is the one that takes the most time; both flash stages are MFMA-bound
+    dom = max((0, 3), key=lambda j: st_ms[j])
+    roof = {
+        "kernel": "flash_kernel<anchor> (stage 1)" if dom == 0 else "flash_kernel<sparse> (stage 3)",
+        "bound": "mfma",
+        "achieved": stage_tflops[dom],
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": stage_tflops[dom] / PEAK_BF16_TFLOPS,
+        "traffic": None,
+        "kernel_ms": st_ms[dom],
+    }
+    rec = {
+        "metric": "anchor_attn_prefill_layer_effective_tflops",
+        "value": (f1 + f2 + f3) / ms_per_step / 1e9,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "n_ctx": n_ctx, "n_q_heads": hq, "n_kv_heads": hkv, "head_dim": D,
+                   "theta": args.theta, "block_size": BS, "step": STEP, "qbar_mode": args.qbar_mode, "seed": args.seed},
+        "sparsity_ratio": ratio,
+        "computed_fraction_of_dense": (f1 + f3) / dense_flops,
+        "stage_ms": {"stage1_anchor": st_ms[0], "pool": st_ms[1], "stage2_select": st_ms[2], "stage3_sparse": st_ms[3]},
+        "stage_tflops": {"stage1": stage_tflops[0], "stage2": stage_tflops[2], "stage3": stage_tflops[3]},
+        "flops": {"F1": f1, "F2": f2, "F3": f3, "dense_causal": dense_flops},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()
