@@ -102,11 +102,11 @@ int check_launch(hipError_t e, const char* who) {
   return AA_OK;
 }
 
-// query rows per work-group = 128 * qb; 2 unless AA_FLASH_QB=1 is exported (tuning knob)
+// query rows per work-group = 128 * qb; 1 unless AA_FLASH_QB=2 is exported (tuning knob)
 int flash_qb() {
   static const int qb = [] {
     const char* e = getenv("AA_FLASH_QB");
-    return (e && e[0] == '1') ? 1 : 2;
+    return (e && e[0] == '2') ? 2 : 1;
   }();
   return qb;
 }

@@ -17,14 +17,14 @@
 // of 16 lanes, lane i receives column i of the 4x16 block whose rows the group's lanes point at).
 //
 // Work-group = 4 waves = 128*QB query rows; keys are consumed 64 at a time through a
-// double-buffered LDS tile (K and V rows padded to 272 bytes).
+// double-buffered LDS tile (K and V rows padded to 304 bytes).
 #include "aa_common.h"
 #include "aa_kernels.h"
 
 namespace aa {
 
 constexpr int kBN = 64;        // keys per LDS tile
-constexpr int kRowStride = 136;  // bf16 per K/V row in LDS (256 B of data + 16 B pad)
+constexpr int kRowStride = 152;  // bf16 per K/V row in LDS: 304 B = 76 dwords keeps both the row-per-lane 16-byte K reads and the transposing V reads free of bank conflicts (measured)
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };

@@ -1,0 +1,145 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the public header declares,
+its host-only helpers compute the documented geometry, and the Python host logic around the
+kernels (layout conversions, argument checks, synthetic inputs) behaves.  No kernel is launched."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from anchor_attn.src.ops import _hip
+from anchor_attn.src.ops import anchor_step_1_2_v2 as st
+from anchor_attn.synthetic import make_qkv, rope_rotate_half, stripe_positions
+
+
+def _declared(repo_root):
+    text = open(os.path.join(repo_root, "include", "anchor_attn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(aa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(repo_root):
+    names = _declared(repo_root)
+    assert len(names) >= 12
+    handle = ctypes.CDLL(_hip.library_path())
+    for n in names:
+        assert hasattr(handle, n), f"{n} is declared in the header but not exported"
+    assert sorted(_hip.EXPORTS) == names, "ctypes signature table and header disagree"
+
+
+def test_host_geometry_helpers():
+    lib = _hip.lib()
+    assert lib.aa_version() >= 1
+    S, bs = 2048, 128
+    for n_bb in (1, 2, 3, 4, 16, 64):
+        want = sum(max(bb * S - 2 * bs, 0) for bb in range(n_bb))
+        assert lib.aa_coords_entries_per_head(n_bb * S, bs, 16) == want
+        assert lib.aa_coords_offset(n_bb, bs, 16) == want
+    assert lib.aa_coords_offset(0, bs, 16) == 0 and lib.aa_coords_offset(1, bs, 16) == 0
+    assert lib.aa_mask_words(1, 32, 131072, 128, 16) * 4 == 32 * 2**20
+    # step 32: big block 4096
+    assert lib.aa_coords_offset(2, bs, 32) == 4096 - 256
+    ws = lib.aa_workspace_bytes(1, 32, 131072, 128, 128, 16)
+    acc = 32 * 131072 * 128 * 4
+    assert acc < ws < acc + 2**30
+    assert lib.aa_workspace_bytes(1, 32, 131072, 64, 128, 16) == 0  # head_dim 64 not supported
+
+
+def test_error_codes_without_touching_the_gpu():
+    """Validation runs before any launch, so bad arguments can be exercised on a CPU-only host."""
+    lib = _hip.lib()
+    buf = ctypes.create_string_buffer(4096 + 64)
+    p = (ctypes.addressof(buf) + 63) & ~63
+    s = (2048 * 128 * 2, 2048 * 128, 128)
+    dense = lambda q, nq, nkv, n, d, qs=s: lib.aa_dense_causal_fwd(q, *qs, p, *s, p, *s, p, *s, 1, nq, nkv, n, d, 0.1, None)
+    assert dense(None, 2, 2, 2048, 128) == 1 and b"q is NULL" in lib.aa_last_error()
+    assert dense(p, 3, 2, 2048, 128) == 1 and b"divide" in lib.aa_last_error()
+    assert dense(p, 2, 2, 2048, 64) == 2 and b"head_dim" in lib.aa_last_error()
+    assert dense(p, 2, 2, 2000, 128) == 2
+    assert dense(p + 2, 2, 2, 2048, 128) == 3 and b"aligned" in lib.aa_last_error()
+    assert dense(p, 2, 2, 2048, 128, qs=(s[0], s[1], 132)) == 3
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1024, None, 1, 2, 2, 2048, 128, 128, 16, 0.1, 12.0, 0, None)
+    assert rc == 1 and b"workspace" in lib.aa_last_error()
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, None)
+    assert rc == 2 and b"multiple" in lib.aa_last_error()
+    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 8, 0.1, 0, None)
+    assert rc == 2 and b"step" in lib.aa_last_error()
+    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 7, None)
+    assert rc == 1 and b"scale_mode" in lib.aa_last_error()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "library_path", lambda: str(tmp_path / "nope.so"))
+    with pytest.raises(_hip.AnchorAttnHipError, match="no fallback"):
+        _hip.lib()
+
+
+def test_cpu_tensors_are_rejected():
+    from anchor_attn.src.ops.anchor_attn_v4 import anchor_attn
+    q = torch.zeros(1, 2, 2048, 128, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="GPU only"):
+        anchor_attn(q, q, q)
+
+
+def test_acc_fragment_order_matches_the_documented_formula():
+    B, H, N, D = 1, 2, 64, 128
+    rows = torch.arange(B * H * N * D, dtype=torch.float32).view(B, H, N, D)
+    frag = torch.empty(B * H * N * D)
+    b, h = np.meshgrid(np.arange(B), np.arange(H), indexing="ij")
+    for hh in range(H):
+        for row in range(N):
+            d = np.arange(D)
+            off = ((((0 * H + hh) * (N // 32) + row // 32) * 4 + d // 32) * 4 + (d % 32) // 8) * 256 \
+                + (((d % 8) // 4) * 32 + row % 32) * 4 + d % 4
+            frag[torch.from_numpy(off)] = rows[0, hh, row]
+    assert torch.equal(st.acc_rows(frag.view(B, H, N, D)), rows)
+
+
+def test_expand_coords_to_reference_layout():
+    lib = _hip.lib()
+    N, bs, step = 3 * 2048, 128, 16
+    per_head = lib.aa_coords_entries_per_head(N, bs, step)
+    coords = torch.full((1, 1, per_head), -7, dtype=torch.int32)
+    counts = torch.tensor([0, 3, 2], dtype=torch.int32).view(1, 1, 3, 1)
+    coords[0, 0, 0:3] = torch.tensor([130, 500, 1900])
+    off2 = lib.aa_coords_offset(2, bs, step)
+    coords[0, 0, off2:off2 + 2] = torch.tensor([128, 3967])
+    tc = st.expand_coords(coords, counts, N, bs, step)
+    assert tc.shape == (1, 1, 3, N)
+    assert tc[0, 0, 1, :4].tolist() == [130, 500, 1900, 0] and tc[0, 0, 2, :3].tolist() == [128, 3967, 0]
+    assert int(tc[0, 0, 0].abs().sum()) == 0 and int((tc < 0).sum()) == 0
+
+
+def test_synthetic_generator_properties():
+    q, k, v, pos = make_qkv(4096, 4, 2, n_stripes=64, seed=9)
+    assert q.shape == (1, 4, 4096, 128) and k.shape == (1, 2, 4096, 128) and q.dtype == torch.bfloat16
+    assert pos.numel() == 64 and pos.min() >= 1 and pos.unique().numel() == 64
+    q2, k2, _, pos2 = make_qkv(4096, 4, 2, n_stripes=64, seed=9)
+    assert torch.equal(q, q2) and torch.equal(k, k2) and torch.equal(pos, pos2)
+    # sink and stripes score far above ordinary keys (shared qbar): ~16 and ~8 nats
+    s = (q[0, 0].float() @ k[0, 0].float().T) / math.sqrt(128)
+    ordinary = torch.ones(4096, dtype=torch.bool)
+    ordinary[0] = False
+    ordinary[pos] = False
+    assert 14 < float(s[:, 0].mean() - s[:, ordinary].mean()) < 18
+    assert 6.5 < float(s[:, pos].mean() - s[:, ordinary].mean()) < 9.5
+    # literal mode: biases vanish
+    ql, kl, _, _ = make_qkv(4096, 4, 2, n_stripes=64, seed=9, qbar_mode="literal")
+    sl = (ql[0, 0].float() @ kl[0, 0].float().T) / math.sqrt(128)
+    assert abs(float(sl[:, 0].mean())) < 0.5
+    # RoPE is a rotation: norms are preserved, position 0 is untouched
+    x = torch.randn(64, 128)
+    y = rope_rotate_half(x, 5e5)
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-4) and torch.equal(y[0], x[0])
+    # relative-position property: <rope(a)_m, rope(b)_n> depends on m - n only
+    a, b = torch.randn(128), torch.randn(128)
+    ra, rb = rope_rotate_half(a.expand(16, 128).clone(), 1e4), rope_rotate_half(b.expand(16, 128).clone(), 1e4)
+    assert abs(float(ra[5] @ rb[3]) - float(ra[12] @ rb[10])) < 1e-3
+    g = torch.Generator().manual_seed(1)
+    pw = stripe_positions(131072, 655, "powerlaw", g)
+    assert pw.numel() == 655 and pw.unique().numel() == 655 and pw.min() >= 1 and pw.max() < 131072
+    assert (pw < 131072 // 4).sum() > 655 * 0.4  # density decays with position (uniform would give 25%)
