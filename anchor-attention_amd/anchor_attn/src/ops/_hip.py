@@ -19,7 +19,8 @@ class AnchorAttnHipError(RuntimeError):
 
 
 def library_path() -> str:
-    return os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+    """The in-tree build; ANCHOR_ATTN_HIP_LIB may point at another build of the same library."""
+    return os.environ.get("ANCHOR_ATTN_HIP_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 
 
 _T3 = [c_void_p, c_int64, c_int64, c_int64]  # pointer + (batch, head, row) element strides

@@ -111,6 +111,20 @@ int flash_qb() {
   return qb;
 }
 
+// AA_FLASH_PIPE=1 selects the software-pipelined 256-row flash kernels (aa_flash2.hip) instead of the
+// default 128-row ones (aa_flash.hip); same results, kept selectable for measurements
+bool flash_pipelined() {
+  static const bool on = [] {
+    const char* e = getenv("AA_FLASH_PIPE");
+    return e && e[0] == '1';
+  }();
+  return on;
+}
+
+hipError_t run_flash(const FlashArgs& a, int mode, hipStream_t stream) {
+  return flash_pipelined() ? launch_flash2(a, mode, stream) : launch_flash(a, mode, flash_qb(), stream);
+}
+
 size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
 struct Workspace {
@@ -187,7 +201,7 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = scale_mode;
-  return check_launch(launch_flash(a, 0, flash_qb(), (hipStream_t)stream), who);
+  return check_launch(run_flash(a, 0, (hipStream_t)stream), who);
 }
 
 int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
@@ -259,7 +273,7 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
-  return check_launch(launch_flash(a, 1, flash_qb(), (hipStream_t)stream), who);
+  return check_launch(run_flash(a, 1, (hipStream_t)stream), who);
 }
 
 int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
@@ -336,7 +350,7 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = n_ctx; a.block_size = 128;  // one "big block": bb is always 0
   a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
-  return check_launch(launch_flash(a, 2, flash_qb(), (hipStream_t)stream), who);
+  return check_launch(run_flash(a, 2, (hipStream_t)stream), who);
 }
 
 }  // extern "C"

@@ -28,6 +28,11 @@ __device__ __forceinline__ float rn16(float a) { return bf16_lo(pack_bf16(a, 0.f
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Work-group barrier for LDS hand-over only: waits for this wave's LDS traffic, then synchronises.
+// Unlike __syncthreads() it does not wait for outstanding global loads, so prefetches issued before
+// the barrier stay in flight across it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // value held by the lane 32 positions away (the two halves of a wave share MFMA columns)
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 

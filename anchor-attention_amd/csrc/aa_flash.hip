@@ -127,6 +127,9 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   const int bb = R0 / S;
   const int wr0 = R0 + wave * 32 * QB;
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
+#ifdef AA_CLOCKS  // timing experiments only: shader-clock and 100 MHz reference stamps
+  const long long aa_c0 = clock64(), aa_w0 = wall_clock64();
+#endif
 
   const __bf16* qp = p.q + b * p.q_sb + hq * p.q_sh;
   const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
@@ -206,29 +209,46 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   for (int i = 0; i < n_tiles; ++i) {
     const int buf = i & 1;
     const int key0 = AA_TILE_KEY0(i);
+#if defined(AA_ABLATE) && (AA_ABLATE == 1 || AA_ABLATE == 3)
+    if (i + 1 < n_tiles && i < 1) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
+#else
     if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
+#endif
 
     // a wave whose rows all lie above this tile (causal) has nothing to do
     const bool wave_active = (MODE == kSparse) || (key0 <= wr0 + 32 * QB - 1);
     if (wave_active) {
       const __bf16* ks_ = sm.t.k[buf] + k_rd;
       // ---- S^T = K Q^T ------------------------------------------------------------------------
+      // K operands are fetched from LDS four k-steps (eight reads) ahead of the MFMAs that use them;
+      // the scheduling fences keep that distance (left alone, the reads sink next to their use and
+      // every MFMA then waits out a full LDS latency).
       floatx16 s[2][QB];
+      bf16x8 ka[8][2];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
+      for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * ks);
+        for (int kb = 0; kb < 2; ++kb) ka[ks][kb] = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * ks);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks + 4 < 8) {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) ka[ks + 4][kb] = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * (ks + 4));
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) {
             if (ks == 0) {
               const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[qb][ks], zero, 0, 0, 0);
+              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], zero, 0, 0, 0);
             } else {
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[qb][ks], s[kb][qb], 0, 0, 0);
+              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], s[kb][qb], 0, 0, 0);
             }
           }
-        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
 
       // ---- masks ------------------------------------------------------------------------------
       if (MODE != kSparse) {
@@ -277,7 +297,11 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
           float pv[16];
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
+#if defined(AA_ABLATE) && (AA_ABLATE == 2)
+            pv[r] = s[kb][qb][r];
+#else
             pv[r] = fast_exp2(s[kb][qb][r] - m_new);
+#endif
             sum += pv[r];
           }
 #pragma unroll
@@ -303,29 +327,49 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
       }
 
       // ---- O^T += V^T P^T ---------------------------------------------------------------------
+      // 16 operand fetches (two transposing reads each), kept four ahead of their MFMAs
       const __bf16* vs_ = sm.t.v[buf] + v_rd;
+      shortx4 vlo[16], vhi[16];
+#define AA_V_SRC(i) (vs_ + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowStride + 32 * ((i) & 3))
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int i = 0; i < 4; ++i) {
+        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i)));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i) + 8 * kRowStride));
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int st = 0; st < 2; ++st)
+      for (int i = 0; i < 16; ++i) {  // i = (kb*2 + st)*4 + db
+        if (i + 4 < 16) {
+          vlo[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4)));
+          vhi[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4) + 8 * kRowStride));
+        }
+        typedef short shortx8 __attribute__((ext_vector_type(8)));
+        const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&av);
+        const int kb = i >> 3, st = (i >> 2) & 1, db = i & 3;
 #pragma unroll
-          for (int db = 0; db < 4; ++db) {
-            const __bf16* src = vs_ + (32 * kb + 16 * st) * kRowStride + 32 * db;
-            const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(src));
-            const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(src + 8 * kRowStride));
-            typedef short shortx8 __attribute__((ext_vector_type(8)));
-            const shortx8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            const bf16x8 a = *reinterpret_cast<const bf16x8*>(&av);
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) acc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[kb][qb][st], acc[db][qb], 0, 0, 0);
-          }
+        for (int qb = 0; qb < QB; ++qb) acc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[kb][qb][st], acc[db][qb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#undef AA_V_SRC
     }
 
+#if defined(AA_ABLATE) && (AA_ABLATE == 3)
+    if (i < 1) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
+#else
     if (i + 1 < n_tiles) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
+#endif
     __syncthreads();
   }
 #undef AA_TILE_KEY0
 
+#ifdef AA_CLOCKS
+  if (MODE == kAnchor && tid == 0 && qblk == n_qblk / 2 && hq == 0 && b == 0) {
+    p.L_out[bh * p.n_ctx + p.n_ctx - 1] = (float)(clock64() - aa_c0);
+    p.L_out[bh * p.n_ctx + p.n_ctx - 2] = (float)(wall_clock64() - aa_w0);
+    p.L_out[bh * p.n_ctx + p.n_ctx - 3] = (float)n_tiles;
+  }
+#endif
   // ---- epilogue --------------------------------------------------------------------------------
   if (MODE == kAnchor) {
 #pragma unroll
