@@ -16,6 +16,12 @@
 // at one head-dim column is fetched with the transposing LDS read ds_read_b64_tr_b16 (within a group
 // of 16 lanes, lane i receives column i of the 4x16 block whose rows the group's lanes point at).
 //
+// The running row max m is subtracted inside the first product: the score accumulators start from
+// -m (a per-lane constant, kept replicated in a 16-register tuple) instead of zero, so the tile
+// arrives as S - m and p = exp2(S - m) needs no subtraction.  Only when some row's max grows (rare
+// after the first tiles) does the wave take a slow path that shifts the tile, re-bases the tuple and
+// rescales the accumulators - which is exact for the lanes whose max did not move (shift 0, factor 1).
+//
 // Work-group = 4 waves = 128*QB query rows; keys are consumed 64 at a time through a
 // double-buffered LDS tile (K and V rows padded to 304 bytes).
 #include "aa_common.h"
@@ -86,8 +92,8 @@ __device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const cha
     } else {
       key = (uint32_t)(key0 + row);
     }
-    r.k[j] = *reinterpret_cast<const u32x4*>(kb + (key * k_row_bytes + col));
-    r.v[j] = *reinterpret_cast<const u32x4*>(vb + (key * v_row_bytes + col));
+    r.k[j] = *reinterpret_cast<const u32x4*>(kb + (__umul24(key, k_row_bytes) + col));
+    r.v[j] = *reinterpret_cast<const u32x4*>(vb + (__umul24(key, v_row_bytes) + col));
   }
 }
 
@@ -198,6 +204,17 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     }
   }
 
+  // m_ref is what the score accumulators are pre-loaded with (negated); it equals m_run except before
+  // the first tile of a fresh row (m_run = -inf, m_ref = 0)
+  float m_ref[QB];
+  floatx16 negm[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_ref[qb] = (MODE == kSparse) ? m_run[qb] : 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negm[qb][r] = -m_ref[qb];
+  }
+
   if (n_tiles > 0) tile_store(tr, sm.t.k[0], sm.t.v[0], tid);
   __syncthreads();
 
@@ -206,8 +223,16 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   // transposing V read: group of 16 lanes covers 16 head-dim columns, lane i points at row i/4, 4 columns from 4*(i%4)
   const int v_rd = (4 * half + ((lane & 15) >> 2)) * kRowStride + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+#ifdef AA_CLOCKS
+  long long aa_ph[6] = {0, 0, 0, 0, 0, 0};
+  long long aa_t = clock64();
+#define AA_STAMP(i) { const long long t_ = clock64(); aa_ph[i] += t_ - aa_t; aa_t = t_; }
+#else
+#define AA_STAMP(i)
+#endif
   for (int i = 0; i < n_tiles; ++i) {
     const int buf = i & 1;
+    AA_STAMP(5)
     const int key0 = AA_TILE_KEY0(i);
 #if defined(AA_ABLATE) && (AA_ABLATE == 1 || AA_ABLATE == 3)
     if (i + 1 < n_tiles && i < 1) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
@@ -215,6 +240,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
 #endif
 
+    AA_STAMP(0)
     // a wave whose rows all lie above this tile (causal) has nothing to do
     const bool wave_active = (MODE == kSparse) || (key0 <= wr0 + 32 * QB - 1);
     if (wave_active) {
@@ -241,8 +267,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) {
             if (ks == 0) {
-              const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], zero, 0, 0, 0);
+              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], negm[qb], 0, 0, 0);
             } else {
               s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], s[kb][qb], 0, 0, 0);
             }
@@ -250,6 +275,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
         __builtin_amdgcn_sched_barrier(0);
       }
 
+      AA_STAMP(1)
       // ---- masks ------------------------------------------------------------------------------
       if (MODE != kSparse) {
         if (key0 + kBN - 1 > wr0) {  // tile touches the diagonal of this wave
@@ -275,10 +301,10 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
             }
       }
 
-      // ---- online soft-max (exp2 domain) ------------------------------------------------------
+      // ---- online soft-max (exp2 domain); s holds S - m_ref ---------------------------------------
       bf16x8 pfrag[2][QB][2];
-      float alpha[QB];
-      bool rescale = false;
+      float mxr[QB];
+      bool moved = false;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         float mx = s[0][qb][0];
@@ -286,11 +312,33 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][qb][r]);
-        mx = fmaxf(mx, xor32(mx));
-        const float m_new = fmaxf(m_run[qb], mx);
-        alpha[qb] = fast_exp2(m_run[qb] - m_new);
-        rescale |= (m_new != m_run[qb]);
-        m_run[qb] = m_new;
+        mxr[qb] = fmaxf(mx, xor32(mx));
+        moved |= (m_ref[qb] + mxr[qb] > m_run[qb]);
+      }
+      if (__any(moved)) {
+        // slow path: some row's max grew.  Lanes whose max did not move get shift 0 and alpha 1 (exact).
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          const float m_new = fmaxf(m_run[qb], m_ref[qb] + mxr[qb]);
+          const float alpha = fast_exp2(m_run[qb] - m_new);
+          const float shift = m_new - m_ref[qb];
+          m_run[qb] = m_new;
+          m_ref[qb] = m_new;
+          l_run[qb] *= alpha;
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][qb][r] -= shift;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) negm[qb][r] = -m_new;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[db][qb][r] *= alpha;
+        }
+      }
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
         float sum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -300,7 +348,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
 #if defined(AA_ABLATE) && (AA_ABLATE == 2)
             pv[r] = s[kb][qb][r];
 #else
-            pv[r] = fast_exp2(s[kb][qb][r] - m_new);
+            pv[r] = fast_exp2(s[kb][qb][r]);
 #endif
             sum += pv[r];
           }
@@ -314,18 +362,10 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
             pfrag[kb][qb][st] = *reinterpret_cast<bf16x8*>(&w);
           }
         }
-        l_run[qb] = l_run[qb] * alpha[qb] + sum;
-      }
-      // multiplying by alpha == 1 is exact, so the rescale is skipped when no lane's max moved
-      if (__any(rescale)) {
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[db][qb][r] *= alpha[qb];
+        l_run[qb] += sum;
       }
 
+      AA_STAMP(2)
       // ---- O^T += V^T P^T ---------------------------------------------------------------------
       // 16 operand fetches (two transposing reads each), kept four ahead of their MFMAs
       const __bf16* vs_ = sm.t.v[buf] + v_rd;
@@ -352,6 +392,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
         __builtin_amdgcn_sched_barrier(0);
       }
 #undef AA_V_SRC
+      AA_STAMP(3)
     }
 
 #if defined(AA_ABLATE) && (AA_ABLATE == 3)
@@ -360,6 +401,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     if (i + 1 < n_tiles) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
 #endif
     __syncthreads();
+    AA_STAMP(4)
   }
 #undef AA_TILE_KEY0
 
@@ -368,6 +410,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     p.L_out[bh * p.n_ctx + p.n_ctx - 1] = (float)(clock64() - aa_c0);
     p.L_out[bh * p.n_ctx + p.n_ctx - 2] = (float)(wall_clock64() - aa_w0);
     p.L_out[bh * p.n_ctx + p.n_ctx - 3] = (float)n_tiles;
+    for (int i = 0; i < 6; ++i) p.L_out[bh * p.n_ctx + p.n_ctx - 4 - i] = (float)aa_ph[i];
   }
 #endif
   // ---- epilogue --------------------------------------------------------------------------------
