@@ -167,8 +167,13 @@ int64_t aa_coords_offset(int big_block, int block_size, int step) {
   return coords_tri(big_block, (int64_t)block_size * step, block_size);
 }
 
-int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int step) {
+static int64_t mask_bit_words(int batch, int n_q_heads, int n_ctx, int block_size, int step) {
   return (int64_t)batch * n_q_heads * (n_ctx / (block_size * step)) * (n_ctx / 128) * 4;
+}
+
+int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int step) {
+  // key bitmask followed by one float32 threshold per pooled row
+  return mask_bit_words(batch, n_q_heads, n_ctx, block_size, step) + (int64_t)batch * n_q_heads * (n_ctx / block_size);
 }
 
 size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int step) {
@@ -235,11 +240,13 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.qbar = (const __bf16*)qbar; a.abar = (const __bf16*)abar;
   a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.mask = mask_ws; a.coords = coords; a.counts = counts;
+  a.thr = reinterpret_cast<float*>(mask_ws + mask_bit_words(batch, n_q_heads, n_ctx, block_size, step));
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
   a.scale2 = (float)((double)sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
+  if ((rc = check_launch(launch_select_thresholds(a, (hipStream_t)stream), who))) return rc;
   if ((rc = check_launch(launch_select_scores(a, (hipStream_t)stream), who))) return rc;
   return check_launch(launch_select_compact(a, (hipStream_t)stream), who);
 }

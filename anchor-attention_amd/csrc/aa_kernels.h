@@ -33,11 +33,13 @@ hipError_t launch_pool(const PoolArgs& a, hipStream_t stream);
 struct SelectArgs {
   const __bf16* qbar; const __bf16* abar;
   const __bf16* k; int64_t k_sb, k_sh, k_sn;
+  float* thr;  // per pooled row: smallest raw dot product that passes the selection test
   uint32_t* mask; int32_t* coords; int32_t* counts; int64_t coords_per_head;
   int batch, n_q_heads, n_kv_heads, n_ctx;
   int big_block, block_size;
   float scale2, theta_log2;
 };
+hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream);
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream);
 hipError_t launch_select_compact(const SelectArgs& a, hipStream_t stream);
 

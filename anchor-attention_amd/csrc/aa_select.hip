@@ -9,6 +9,11 @@
 //           In the 32x32 accumulator a lane holds one key column; OR-ing its registers over the pooled
 //           rows of a big block and a wave ballot give a 32-bit key mask per (q head, big block, key
 //           block) with no LDS and no atomics.
+//  thresholds  the as-specified test "float(bf16(raw * scale)) + theta >= anchor" is monotone in the raw
+//           float32 dot product, so for every pooled row there is one float32 number x* with
+//           "test passes  <=>  raw >= x*".  A tiny kernel finds x* per pooled row by bisection over
+//           the ordered float32 bit patterns, evaluating the test exactly as written; the score
+//           kernel's epilogue is then a single compare per element.
 //  compact  one wave per (batch, q head, big block) turns that big block's mask row into an ascending
 //           index list with popcounts and a wave prefix sum.
 #include "aa_common.h"
@@ -59,6 +64,42 @@ hipError_t launch_pool(const PoolArgs& a, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// Smallest float32 x with  float(bf16(x * scale2)) + theta >= anchor  (NaN if there is none).
+__device__ __forceinline__ bool select_test(const float x, const float scale2, const float theta, const float anchor) {
+  const float sc = rn16(x * scale2);  // float32 product, then bf16
+  return (sc + theta) >= anchor;      // float32 add and compare, non-strict
+}
+__device__ __forceinline__ float ordered_to_float(const uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);  // monotone bijection uint32 -> float32
+}
+
+__global__ void __launch_bounds__(256) select_threshold_kernel(const __bf16* __restrict__ abar, float* __restrict__ thr, const int n,
+                                                                const float scale2, const float theta) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float anchor = bf16_lo(reinterpret_cast<const uint16_t*>(abar)[i]);
+  // ordered keys: 0x007fffff <-> -inf, 0xff800000 <-> +inf (NaNs lie outside that range)
+  uint32_t lo = 0x007fffffu, hi = 0xff800000u;
+  float out;
+  if (!select_test(ordered_to_float(hi), scale2, theta, anchor)) {
+    out = __uint_as_float(0x7fc00000u);  // no float passes: NaN compares false with everything
+  } else {
+    while (lo < hi) {  // invariant: test(hi) is true
+      const uint32_t mid = lo + ((hi - lo) >> 1);
+      if (select_test(ordered_to_float(mid), scale2, theta, anchor)) hi = mid; else lo = mid + 1;
+    }
+    out = ordered_to_float(hi);
+  }
+  thr[i] = out;
+}
+
+hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
+  const int n = a.batch * a.n_q_heads * (a.n_ctx / a.block_size);
+  hipLaunchKernelGGL(select_threshold_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.abar, a.thr, n, a.scale2, a.theta_log2);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
 // STEP = pooled rows per big block (16 or 32); 32 / STEP (head, big block) items share one MFMA.
 template <int STEP>
 __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) {
@@ -89,29 +130,28 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
     for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
   }
 
-  for (int grp = wave; grp < n_groups; grp += 4) {
-    // A operand: row c32 of this MFMA is pooled row (c32 % STEP) of item grp*kItems + c32/STEP
+  // operands of one group: A = 32 pooled query rows (row c32 of the MFMA is pooled row c32 % STEP of item
+  // grp*kItems + c32/STEP) and the raw-score thresholds of the accumulator rows this lane holds
+  // (row i = 8*(r/4) + 4*half + r%4)
+  auto load_group = [&](const int grp, bf16x8 (&a)[8], float (&thr)[16]) {
     const int item_a = min(grp * kItems + c32 / STEP, n_items - 1);
     const int hq_a = kvh * group + item_a % group;
     const int bb_a = bb_min + item_a / group;
     const __bf16* qrow = p.qbar + (((int64_t)b * p.n_q_heads + hq_a) * n_pr + bb_a * STEP + c32 % STEP) * 128 + 8 * half;
-    bf16x8 a[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks);
-
-    // thresholds for the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
-    float thr[16];
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
       const int i0 = 8 * rq + 4 * half;
       const int item = min(grp * kItems + i0 / STEP, n_items - 1);
       const int hq = kvh * group + item % group;
       const int bb = bb_min + item / group;
-      const uint2 w = *reinterpret_cast<const uint2*>(p.abar + ((int64_t)b * p.n_q_heads + hq) * n_pr + bb * STEP + i0 % STEP);
-      thr[4 * rq + 0] = bf16_lo(w.x); thr[4 * rq + 1] = bf16_hi(w.x);
-      thr[4 * rq + 2] = bf16_lo(w.y); thr[4 * rq + 3] = bf16_hi(w.y);
+      const floatx4 w = *reinterpret_cast<const floatx4*>(p.thr + ((int64_t)b * p.n_q_heads + hq) * n_pr + bb * STEP + i0 % STEP);
+      thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
+      thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
     }
-
+  };
+  auto compute_group = [&](const int grp, const bf16x8 (&a)[8], const float (&thr)[16]) {
     uint32_t words[kItems][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -124,11 +164,7 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
 #pragma unroll
       for (int it = 0; it < kItems; ++it) hit[it] = false;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float sc = rn16(c[r] * p.scale2);          // float32 product, then bf16
-        const bool pass = (sc + p.theta_log2) >= thr[r];  // float32 add and compare, non-strict
-        hit[(8 * (r >> 2)) / STEP] |= pass;                // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
-      }
+      for (int r = 0; r < 16; ++r) hit[(8 * (r >> 2)) / STEP] |= (c[r] >= thr[r]);  // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
 #pragma unroll
       for (int it = 0; it < kItems; ++it) {
         const uint64_t m = __ballot(hit[it]);
@@ -147,6 +183,21 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
         }
       }
     }
+  };
+
+  // two operand sets: the next group's operands are on their way from L2 while this one is multiplied
+  bf16x8 a0[8], a1[8];
+  float thr0[16], thr1[16];
+  int grp = wave;
+  if (grp < n_groups) load_group(grp, a0, thr0);
+  while (grp < n_groups) {
+    if (grp + 4 < n_groups) load_group(grp + 4, a1, thr1);
+    compute_group(grp, a0, thr0);
+    grp += 4;
+    if (grp >= n_groups) break;
+    if (grp + 4 < n_groups) load_group(grp + 4, a0, thr0);
+    compute_group(grp, a1, thr1);
+    grp += 4;
   }
 }
 

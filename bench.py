@@ -24,6 +24,12 @@ for _p in (ROOT, os.path.join(ROOT, "anchor-attention_amd")):
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/hbm_traffic_*.md); a counter
+# run cannot be made from inside this script, so the figure is carried here for the workload it was taken on
+MEASURED_TRAFFIC_BYTES = {
+    "config2_llama8b_128k": {0: 4.39e9, 3: 4.44e9},  # dominant-kernel index -> bytes (stage 1, stage 3)
+}
+
 WORKLOADS = {
     # name: (n_ctx, hq, hkv, rope_base, n_stripes, stripe_dist)
     "config0_llama8b_4k": (4096, 32, 8, 5e5, 64, "uniform"),
@@ -124,6 +130,9 @@ def main():
     ap.add_argument("--qbar-mode", default="shared", choices=["shared", "literal"])
     ap.add_argument("--seed", type=int, default=2024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 1 GiB device copies (a kernel of known traffic) so that rocprofv3 "
+                         "FETCH_SIZE/WRITE_SIZE readings of the attention kernels can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the operator is embarrassingly parallel over KV-head "
@@ -140,6 +149,12 @@ def main():
     sm = 1.0 / math.sqrt(D)
     q, k, v = make_inputs(args.workload, args.seed, args.qbar_mode, dev)
     out = torch.empty_like(q)
+    if args.calibrate_copy:
+        src = torch.ones(2**28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        del src, dst
     torch.cuda.synchronize()
 
     # ---- timed region: K calls of the public operator -----------------------------------------
@@ -191,7 +206,7 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": stage_tflops[dom] / PEAK_BF16_TFLOPS,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom) if (args.theta == 12.0 and args.qbar_mode == "shared") else None,
         "kernel_ms": st_ms[dom],
     }
     rec = {

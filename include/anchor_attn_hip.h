@@ -53,7 +53,8 @@ const char* aa_last_error(void);
 int64_t aa_coords_entries_per_head(int n_ctx, int block_size, int step);
 int64_t aa_coords_offset(int big_block, int block_size, int step);
 
-/* Number of uint32 words of the stage-2 key bitmask: [batch, n_q_heads, n_ctx/S, n_ctx/128, 4]. */
+/* Number of uint32 words of the stage-2 scratch: the key bitmask [batch, n_q_heads, n_ctx/S, n_ctx/128, 4]
+ * followed by one float32 selection threshold per pooled query row [batch, n_q_heads, n_ctx/block_size]. */
 int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int step);
 
 /* Bytes of scratch aa_anchor_attn_fwd() needs (M, L, Acc, pooled q, pooled anchors, bitmask,

@@ -39,7 +39,7 @@ def test_host_geometry_helpers():
         assert lib.aa_coords_entries_per_head(n_bb * S, bs, 16) == want
         assert lib.aa_coords_offset(n_bb, bs, 16) == want
     assert lib.aa_coords_offset(0, bs, 16) == 0 and lib.aa_coords_offset(1, bs, 16) == 0
-    assert lib.aa_mask_words(1, 32, 131072, 128, 16) * 4 == 32 * 2**20
+    assert lib.aa_mask_words(1, 32, 131072, 128, 16) * 4 == 32 * 2**20 + 32 * 1024 * 4  # bitmask + per-pooled-row thresholds
     # step 32: big block 4096
     assert lib.aa_coords_offset(2, bs, 32) == 4096 - 256
     ws = lib.aa_workspace_bytes(1, 32, 131072, 128, 128, 16)
