@@ -32,6 +32,7 @@ namespace aa {
 constexpr int kBN = 64;        // keys per LDS tile
 constexpr int kRowStride = 152;  // bf16 per K/V row in LDS: 304 B = 76 dwords keeps both the row-per-lane 16-byte K reads and the transposing V reads free of bank conflicts (measured)
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
+constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
 
@@ -40,7 +41,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
 
-template <int QB>
+template <int QB, bool WITH_IDX>
 struct FlashSmem {
   union {
     struct {
@@ -49,6 +50,7 @@ struct FlashSmem {
     } t;
     __bf16 os[4][32 * QB * kOsStride];  // epilogue staging, reuses the tile space
   };
+  int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
 };
 
 __device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale, const bool bf16_chain) {
@@ -76,11 +78,12 @@ struct TileRegs {
 };
 
 // Thread t moves 16-byte chunk (t & 15) of tile rows (t >> 4) + 16*j, j = 0..3, for K and for V.
-// `kb`/`vb` are the wave-uniform head bases; row offsets are 32-bit byte offsets.
+// `kb`/`vb` are the wave-uniform head bases; row offsets are 32-bit byte offsets.  Gathered tiles take
+// their row numbers from the LDS window of the index list (a dependent global load per tile would put a
+// full memory latency on the critical path of every tile).
 template <int MODE>
 __device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const char* vb, const uint32_t k_row_bytes,
-                                          const uint32_t v_row_bytes, const int key0, const int tid, const int32_t* cbase,
-                                          const int cnt) {
+                                          const uint32_t v_row_bytes, const int key0, const int tid, const int32_t* idx_win) {
   const int row0 = tid >> 4;
   const uint32_t col = (tid & 15) * 16;
 #pragma unroll
@@ -88,7 +91,7 @@ __device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const cha
     const int row = row0 + 16 * j;
     uint32_t key;
     if (MODE == kSparse) {
-      key = (key0 + row < cnt) ? (uint32_t)cbase[key0 + row] : 0u;  // tail lanes read row 0, masked later
+      key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
     } else {
       key = (uint32_t)(key0 + row);
     }
@@ -109,7 +112,7 @@ __device__ __forceinline__ void tile_store(const TileRegs& r, __bf16* ks, __bf16
 
 template <int QB, int MODE>
 __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const FlashArgs p) {
-  __shared__ __attribute__((aligned(16))) FlashSmem<QB> sm;
+  __shared__ __attribute__((aligned(16))) FlashSmem<QB, MODE == kSparse> sm;
   constexpr int BM = 128 * QB;
 
   const int tid = threadIdx.x;
@@ -127,13 +130,16 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   const int kvh = vid % p.n_kv_heads;
   const int b = vid / p.n_kv_heads;
   const int hq = kvh * group + g;
-  if (MODE != kSparse) qblk = n_qblk - 1 - qblk;  // longest rows first
+  qblk = n_qblk - 1 - qblk;  // longest rows first (later big blocks also carry the longest index lists)
   const int R0 = qblk * BM;
   const int S = p.big_block;
   const int bb = R0 / S;
   const int wr0 = R0 + wave * 32 * QB;
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 #ifdef AA_CLOCKS  // timing experiments only: shader-clock and 100 MHz reference stamps
+#ifndef AA_CLOCKS_QBLK
+#define AA_CLOCKS_QBLK (n_qblk / 2)
+#endif
   const long long aa_c0 = clock64(), aa_w0 = wall_clock64();
 #endif
 
@@ -158,8 +164,23 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   // first key (anchor, dense) or first list position (sparse) of tile i
 #define AA_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
 
+  // sparse mode: list positions [w0, w0 + kIdxWin) -> LDS (zeros past the count)
+  auto fill_index_window = [&](const int w0) {
+    const int pos = w0 + 4 * tid;
+    int4 v = {0, 0, 0, 0};
+    if (pos < cnt) v = *reinterpret_cast<const int4*>(cbase + pos);  // lists start 16-byte aligned; capacity is a multiple of 4
+    if (pos + 1 >= cnt) v.y = 0;
+    if (pos + 2 >= cnt) v.z = 0;
+    if (pos + 3 >= cnt) v.w = 0;
+    *reinterpret_cast<int4*>(&sm.idx[4 * tid]) = v;
+  };
+  if (MODE == kSparse && n_tiles > 0) {
+    fill_index_window(0);
+    __syncthreads();
+  }
+
   TileRegs tr;
-  if (n_tiles > 0) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(0), tid, cbase, cnt);
+  if (n_tiles > 0) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(0), tid, sm.idx);
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
   bf16x8 qreg[QB][8];
@@ -234,10 +255,15 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     const int buf = i & 1;
     AA_STAMP(5)
     const int key0 = AA_TILE_KEY0(i);
+    if (MODE == kSparse && i + 1 < n_tiles && ((i + 1) & (kIdxWin / kBN - 1)) == 0) {
+      // tile i+1 opens the next window; everyone finished reading the old one before the last barrier
+      fill_index_window((i + 1) * kBN);
+      __syncthreads();
+    }
 #if defined(AA_ABLATE) && (AA_ABLATE == 1 || AA_ABLATE == 3)
-    if (i + 1 < n_tiles && i < 1) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
+    if (i + 1 < n_tiles && i < 1) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, sm.idx);
 #else
-    if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, cbase, cnt);
+    if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, sm.idx);
 #endif
 
     AA_STAMP(0)
@@ -406,7 +432,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
 #undef AA_TILE_KEY0
 
 #ifdef AA_CLOCKS
-  if (MODE == kAnchor && tid == 0 && qblk == n_qblk / 2 && hq == 0 && b == 0) {
+  if (MODE != kDense && tid == 0 && qblk == AA_CLOCKS_QBLK && hq == 0 && b == 0) {
     p.L_out[bh * p.n_ctx + p.n_ctx - 1] = (float)(clock64() - aa_c0);
     p.L_out[bh * p.n_ctx + p.n_ctx - 2] = (float)(wall_clock64() - aa_w0);
     p.L_out[bh * p.n_ctx + p.n_ctx - 3] = (float)n_tiles;

@@ -228,7 +228,7 @@ __global__ void __launch_bounds__(256, 1) flash2_kernel(const FlashArgs p) {
   const int kvh = vid % p.n_kv_heads;
   const int b = vid / p.n_kv_heads;
   const int hq = kvh * group + g;
-  if (MODE != kSparse) qblk = n_qblk - 1 - qblk;  // longest rows first
+  qblk = n_qblk - 1 - qblk;  // longest rows first (later big blocks also carry the longest index lists)
   const int R0 = qblk * BM;
   const int S = p.big_block;
   const int bb = R0 / S;

@@ -2,10 +2,11 @@
 //
 //  pool     qbar = bf16(mean of 128 raw query rows), abar = bf16(mean of 128 anchors); float32 sums in
 //           ascending row order so the result is reproducible bit for bit.
-//  scores   K-stationary: one work-group per (batch, KV head, 128-key tile) keeps the key tile in
-//           registers as the MFMA B operand and streams the pooled query rows of EVERY query head of
-//           the KV group and EVERY later big block past it (A operand, 32 pooled rows per MFMA).  Each
-//           K row is thus read once per KV head instead of once per (query head, big block).
+//  scores   K-stationary: one work-group per (batch, KV head, 512 keys); each of its four waves keeps a
+//           128-key tile in registers as the MFMA B operand, and the pooled query rows of EVERY query
+//           head of the KV group and EVERY later big block stream past them (A operand, 32 pooled rows
+//           per MFMA, staged once per work-group in LDS).  Each K row is thus read once per KV head
+//           instead of once per (query head, big block).
 //           In the 32x32 accumulator a lane holds one key column; OR-ing its registers over the pooled
 //           rows of a big block and a wave ballot give a 32-bit key mask per (q head, big block, key
 //           block) with no LDS and no atomics.
@@ -101,109 +102,138 @@ hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
 
 // ------------------------------------------------------------------------------------------------
 // STEP = pooled rows per big block (16 or 32); 32 / STEP (head, big block) items share one MFMA.
+// Work-group = 4 waves = 512 keys: wave w keeps key tile 4*T + w in registers (MFMA B operand) and all
+// four waves multiply the same stream of pooled-query groups, which is staged once per work-group in
+// LDS (double-buffered, one barrier per group) together with the groups' thresholds.
+constexpr int kARowStride = 136;  // bf16 per staged pooled-query row: 272 B, conflict-free for row-per-lane 16-byte reads
+
 template <int STEP>
 __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) {
   constexpr int kItems = 32 / STEP;
-  const int t = blockIdx.x;  // key tile (128 keys)
+  __shared__ __attribute__((aligned(16))) __bf16 a_lds[2][32 * kARowStride];
+  __shared__ __attribute__((aligned(16))) float thr_lds[2][32];
+
+  const int T = blockIdx.x;  // key super-tile (512 keys)
   const int kvh = blockIdx.y, b = blockIdx.z;
   const int n_bb = p.n_ctx / p.big_block;
   const int n_t = p.n_ctx / 128;
   const int n_pr = n_t;  // pooled rows per head (block_size == 128)
-  // tile t is a candidate for big block bb iff 1 <= t <= STEP*bb - 2
-  if (t == 0) return;
-  const int bb_min = (t + 2 + STEP - 1) / STEP;
-  if (bb_min >= n_bb) return;
-  const int group = p.n_q_heads / p.n_kv_heads;
-  const int n_items = group * (n_bb - bb_min);
-  const int n_groups = (n_items + kItems - 1) / kItems;
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, c32 = lane & 31;
+
+  // key tile t is a candidate for big block bb iff 1 <= t <= STEP*bb - 2, i.e. bb >= (t + 2 + STEP - 1) / STEP
+  const int tw = 4 * T + wave;                                   // this wave's key tile
+  const int bb_min_w = tw == 0 ? n_bb : (tw + 2 + STEP - 1) / STEP;  // tile 0 is never a candidate
+  const int t_first = T == 0 ? 1 : 4 * T;                         // first candidate tile of the work-group
+  const int bb_lo = (t_first + 2 + STEP - 1) / STEP;              // smallest big block any wave needs
+  if (bb_lo >= n_bb) return;
+  const int group = p.n_q_heads / p.n_kv_heads;
+  const int n_items = group * (n_bb - bb_lo);
+  const int n_groups = (n_items + kItems - 1) / kItems;
 
   const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
   bf16x8 kreg[4][8];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
-    const __bf16* row = kp + (int64_t)(t * 128 + 32 * kb + c32) * p.k_sn + 8 * half;
+    const __bf16* row = kp + (int64_t)(tw * 128 + 32 * kb + c32) * p.k_sn + 8 * half;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
   }
 
-  // operands of one group: A = 32 pooled query rows (row c32 of the MFMA is pooled row c32 % STEP of item
-  // grp*kItems + c32/STEP) and the raw-score thresholds of the accumulator rows this lane holds
-  // (row i = 8*(r/4) + 4*half + r%4)
-  auto load_group = [&](const int grp, bf16x8 (&a)[8], float (&thr)[16]) {
-    const int item_a = min(grp * kItems + c32 / STEP, n_items - 1);
-    const int hq_a = kvh * group + item_a % group;
-    const int bb_a = bb_min + item_a / group;
-    const __bf16* qrow = p.qbar + (((int64_t)b * p.n_q_heads + hq_a) * n_pr + bb_a * STEP + c32 % STEP) * 128 + 8 * half;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(qrow + 16 * ks);
-#pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      const int i0 = 8 * rq + 4 * half;
-      const int item = min(grp * kItems + i0 / STEP, n_items - 1);
-      const int hq = kvh * group + item % group;
-      const int bb = bb_min + item / group;
-      const floatx4 w = *reinterpret_cast<const floatx4*>(p.thr + ((int64_t)b * p.n_q_heads + hq) * n_pr + bb * STEP + i0 % STEP);
-      thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
-      thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
+  // staging: thread t carries 32 bytes (chunks 2*(t&7), 2*(t&7)+1) of pooled row t>>3 of the group; row r of a
+  // group is pooled row (r % STEP) of item grp*kItems + r/STEP; threads 0..31 also carry the row's threshold
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 st0, st1;
+  float st_thr = 0.f;
+  auto stage_load = [&](const int grp) {
+    const int r = tid >> 3;
+    const int item = min(grp * kItems + r / STEP, n_items - 1);
+    const int64_t prow = ((int64_t)b * p.n_q_heads + kvh * group + item % group) * n_pr + (bb_lo + item / group) * STEP + r % STEP;
+    const __bf16* src = p.qbar + prow * 128 + 16 * (tid & 7);
+    st0 = *reinterpret_cast<const u32x4*>(src);
+    st1 = *reinterpret_cast<const u32x4*>(src + 8);
+    if (tid < 32) {
+      const int item2 = min(grp * kItems + tid / STEP, n_items - 1);
+      st_thr = p.thr[((int64_t)b * p.n_q_heads + kvh * group + item2 % group) * n_pr + (bb_lo + item2 / group) * STEP + tid % STEP];
     }
   };
-  auto compute_group = [&](const int grp, const bf16x8 (&a)[8], const float (&thr)[16]) {
-    uint32_t words[kItems][4];
+  auto stage_store = [&](const int buf) {
+    __bf16* dst = &a_lds[buf][(tid >> 3) * kARowStride + 16 * (tid & 7)];
+    *reinterpret_cast<u32x4*>(dst) = st0;
+    *reinterpret_cast<u32x4*>(dst + 8) = st1;
+    if (tid < 32) thr_lds[buf][tid] = st_thr;
+  };
+
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+
+  for (int grp = 0; grp < n_groups; ++grp) {
+    const int buf = grp & 1;
+    if (grp + 1 < n_groups) stage_load(grp + 1);
+
+    // does this wave's key tile belong to the candidate range of either item of the group?
+    bool item_ok[kItems];
+    bool any_ok = false;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      floatx16 c;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) c[r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c, 0, 0, 0);
-      bool hit[kItems];
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) hit[it] = false;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) hit[(8 * (r >> 2)) / STEP] |= (c[r] >= thr[r]);  // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) {
-        const uint64_t m = __ballot(hit[it]);
-        words[it][kb] = (uint32_t)m | (uint32_t)(m >> 32);  // both halves of the wave hold the same keys
-      }
+    for (int it = 0; it < kItems; ++it) {
+      const int item = grp * kItems + it;
+      item_ok[it] = item < n_items && (bb_lo + item / group) >= bb_min_w;
+      any_ok |= item_ok[it];
     }
-    if (lane == 0) {
+    if (any_ok) {
+      bf16x8 a[8];
+      const __bf16* arow = &a_lds[buf][c32 * kARowStride + 8 * half];
 #pragma unroll
-      for (int it = 0; it < kItems; ++it) {
-        const int item = grp * kItems + it;
-        if (item < n_items) {
-          const int hq = kvh * group + item % group;
-          const int bb = bb_min + item / group;
-          uint4 w = {words[it][0], words[it][1], words[it][2], words[it][3]};
-          *reinterpret_cast<uint4*>(p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + t) * 4) = w;
+      for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(arow + 16 * ks);
+      // raw-score thresholds of the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
+      float thr[16];
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const floatx4 w = *reinterpret_cast<const floatx4*>(&thr_lds[buf][8 * rq + 4 * half]);
+        thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
+        thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
+      }
+      uint32_t words[kItems][4];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        floatx16 c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kreg[kb][0], zero, 0, 0, 0);
+#pragma unroll
+        for (int ks = 1; ks < 8; ++ks) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c, 0, 0, 0);
+        bool hit[kItems];
+#pragma unroll
+        for (int it = 0; it < kItems; ++it) hit[it] = false;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) hit[(8 * (r >> 2)) / STEP] |= (c[r] >= thr[r]);  // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
+#pragma unroll
+        for (int it = 0; it < kItems; ++it) {
+          const uint64_t m = __ballot(hit[it]);
+          words[it][kb] = (uint32_t)m | (uint32_t)(m >> 32);  // both halves of the wave hold the same keys
+        }
+      }
+      if (lane == 0) {
+#pragma unroll
+        for (int it = 0; it < kItems; ++it) {
+          if (item_ok[it]) {
+            const int item = grp * kItems + it;
+            const int hq = kvh * group + item % group;
+            const int bb = bb_lo + item / group;
+            uint4 w = {words[it][0], words[it][1], words[it][2], words[it][3]};
+            *reinterpret_cast<uint4*>(p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + tw) * 4) = w;
+          }
         }
       }
     }
-  };
-
-  // two operand sets: the next group's operands are on their way from L2 while this one is multiplied
-  bf16x8 a0[8], a1[8];
-  float thr0[16], thr1[16];
-  int grp = wave;
-  if (grp < n_groups) load_group(grp, a0, thr0);
-  while (grp < n_groups) {
-    if (grp + 4 < n_groups) load_group(grp + 4, a1, thr1);
-    compute_group(grp, a0, thr0);
-    grp += 4;
-    if (grp >= n_groups) break;
-    if (grp + 4 < n_groups) load_group(grp + 4, a0, thr0);
-    compute_group(grp, a1, thr1);
-    grp += 4;
+    if (grp + 1 < n_groups) stage_store(buf ^ 1);
+    __syncthreads();
   }
 }
 
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
   const int step = a.big_block / a.block_size;
-  const dim3 grid(a.n_ctx / 128, a.n_kv_heads, a.batch);
+  const dim3 grid(a.n_ctx / 512, a.n_kv_heads, a.batch);
   if (step == 16) hipLaunchKernelGGL(select_scores_kernel<16>, grid, dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(select_scores_kernel<32>, grid, dim3(256), 0, stream, a);
   return hipGetLastError();
