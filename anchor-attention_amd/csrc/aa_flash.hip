@@ -23,14 +23,21 @@
 // rescales the accumulators - which is exact for the lanes whose max did not move (shift 0, factor 1).
 //
 // Work-group = 4 waves = 128*QB query rows; keys are consumed 64 at a time through a
-// double-buffered LDS tile (K and V rows padded to 304 bytes).
+// double-buffered LDS tile that the memory system fills directly (global_load_lds_dwordx4: no staging
+// registers, no LDS store instructions).  Such a load writes lane L's 16 bytes at M0 + 16*L, so LDS rows
+// are unpadded 256 bytes; bank conflicts are avoided by XOR-swizzling the 16-byte chunks of a row, which
+// costs nothing on the load side (a lane simply fetches the chunk that belongs in its slot):
+//   K row r, chunk c  ->  slot c ^ (r & 15)          (row-per-lane 16-byte reads)
+//   V row r, chunk c  ->  slot c ^ ((r & 7) << 1)    (transposing 8-byte reads)
+// Both choices measure conflict-free for their read pattern (and each is 2-way conflicted for the other's).
 #include "aa_common.h"
 #include "aa_kernels.h"
 
 namespace aa {
 
 constexpr int kBN = 64;        // keys per LDS tile
-constexpr int kRowStride = 152;  // bf16 per K/V row in LDS: 304 B = 76 dwords keeps both the row-per-lane 16-byte K reads and the transposing V reads free of bank conflicts (measured)
+constexpr int kRowBytes = 256;   // one K/V row in LDS (128 bf16, unpadded, chunks swizzled)
+constexpr int kTileBytes = kBN * kRowBytes;
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
 constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
 
@@ -45,8 +52,8 @@ template <int QB, bool WITH_IDX>
 struct FlashSmem {
   union {
     struct {
-      __bf16 k[2][kBN * kRowStride];
-      __bf16 v[2][kBN * kRowStride];
+      char k[2][kTileBytes];
+      char v[2][kTileBytes];
     } t;
     __bf16 os[4][32 * QB * kOsStride];  // epilogue staging, reuses the tile space
   };
@@ -71,21 +78,25 @@ __device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale
   return *reinterpret_cast<const bf16x8*>(&packed);
 }
 
-// Registers that carry one K/V tile from global memory to LDS.
-struct TileRegs {
-  u32x4 k[4];
-  u32x4 v[4];
-};
+typedef __attribute__((address_space(3))) char lds_char;
+__device__ __forceinline__ uint32_t lds_addr(const void* p) { return (uint32_t)(uintptr_t)(lds_char*)p; }
 
-// Thread t moves 16-byte chunk (t & 15) of tile rows (t >> 4) + 16*j, j = 0..3, for K and for V.
-// `kb`/`vb` are the wave-uniform head bases; row offsets are 32-bit byte offsets.  Gathered tiles take
-// their row numbers from the LDS window of the index list (a dependent global load per tile would put a
-// full memory latency on the critical path of every tile).
+// 64 lanes x 16 bytes, global -> LDS without passing through registers: lane L's bytes land at
+// lds_dst + 16*L (lds_dst is wave-uniform and travels in M0).  Completion is tracked by vmcnt.
+__device__ __forceinline__ void load16_to_lds(const char* base, const uint32_t byte_off, const uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_dst), "v"(byte_off), "s"(base) : "memory");
+}
+
+// One K/V tile: wave w fills LDS rows 16*j + 4*w .. +3 (j = 0..3), i.e. thread t brings the chunk that belongs in
+// slot (t & 15) of row (t >> 4) + 16*j.  `kb`/`vb` are the wave-uniform head bases, `k_col`/`v_col` the byte
+// offset of this thread's (swizzled) chunk inside a row, `lds_k`/`lds_v` the LDS address of row 4*w of the
+// destination tile.  Gathered tiles take their row numbers from the LDS window of the index list (a dependent
+// global load per tile would put a full memory latency on the critical path of every tile).
 template <int MODE>
-__device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const char* vb, const uint32_t k_row_bytes,
-                                          const uint32_t v_row_bytes, const int key0, const int tid, const int32_t* idx_win) {
+__device__ __forceinline__ void tile_fetch(const char* kb, const char* vb, const uint32_t k_row_bytes, const uint32_t v_row_bytes,
+                                           const uint32_t k_col, const uint32_t v_col, const int key0, const int tid,
+                                           const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v) {
   const int row0 = tid >> 4;
-  const uint32_t col = (tid & 15) * 16;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = row0 + 16 * j;
@@ -95,18 +106,8 @@ __device__ __forceinline__ void tile_load(TileRegs& r, const char* kb, const cha
     } else {
       key = (uint32_t)(key0 + row);
     }
-    r.k[j] = *reinterpret_cast<const u32x4*>(kb + (__umul24(key, k_row_bytes) + col));
-    r.v[j] = *reinterpret_cast<const u32x4*>(vb + (__umul24(key, v_row_bytes) + col));
-  }
-}
-
-__device__ __forceinline__ void tile_store(const TileRegs& r, __bf16* ks, __bf16* vs, const int tid) {
-  const int row0 = tid >> 4, c = tid & 15;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int off = (row0 + 16 * j) * kRowStride + 8 * c;
-    *reinterpret_cast<u32x4*>(ks + off) = r.k[j];
-    *reinterpret_cast<u32x4*>(vs + off) = r.v[j];
+    load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
+    load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
   }
 }
 
@@ -179,8 +180,11 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     __syncthreads();
   }
 
-  TileRegs tr;
-  if (n_tiles > 0) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(0), tid, sm.idx);
+  // this thread's chunk of a row (swizzled: see the top of the file) and the wave's slice of the LDS tiles
+  const uint32_t k_col = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15)) * 16u;
+  const uint32_t v_col = (uint32_t)((tid & 15) ^ (((tid >> 4) & 7) << 1)) * 16u;
+  const uint32_t lds_k0 = lds_addr(sm.t.k[0]) + wave * 4 * kRowBytes, lds_v0 = lds_addr(sm.t.v[0]) + wave * 4 * kRowBytes;
+  if (n_tiles > 0) tile_fetch<MODE>(kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0);
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
   bf16x8 qreg[QB][8];
@@ -236,13 +240,23 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     for (int r = 0; r < 16; ++r) negm[qb][r] = -m_ref[qb];
   }
 
-  if (n_tiles > 0) tile_store(tr, sm.t.k[0], sm.t.v[0], tid);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
   __syncthreads();
 
-  // per-lane LDS offsets (in bf16 elements)
-  const int k_rd = c32 * kRowStride + 8 * half;  // K row c32 (+32*kb), columns 8*half (+16*ks)
-  // transposing V read: group of 16 lanes covers 16 head-dim columns, lane i points at row i/4, 4 columns from 4*(i%4)
-  const int v_rd = (4 * half + ((lane & 15) >> 2)) * kRowStride + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  // per-lane LDS byte offsets.  K: row c32 (+32*kb), chunk 2*ks + half, swizzled with the row's low four bits.
+  uint32_t k_rd[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) k_rd[ks] = c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  // transposing V read i: a group of 16 lanes covers 16 head-dim columns; lane points at row r0 = 4*half + (lane%16)/4
+  // (+ multiples of 8, which leave r0 = row & 7 alone), bf16 columns 32*(i&3) + 16*((lane>>4)&1) + 4*(lane&3): chunk
+  // 4*(i&3) + y0 with y0 < 4, swizzled with r0 << 1 -> one offset per value of i & 3
+  uint32_t v_rd[4];
+  {
+    const int r0 = 4 * half + ((lane & 15) >> 2);
+    const int y0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) v_rd[m] = r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
+  }
 
 #ifdef AA_CLOCKS
   long long aa_ph[6] = {0, 0, 0, 0, 0, 0};
@@ -260,17 +274,16 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
       fill_index_window((i + 1) * kBN);
       __syncthreads();
     }
-#if defined(AA_ABLATE) && (AA_ABLATE == 1 || AA_ABLATE == 3)
-    if (i + 1 < n_tiles && i < 1) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, sm.idx);
-#else
-    if (i + 1 < n_tiles) tile_load<MODE>(tr, kbase, vbase, k_row_bytes, v_row_bytes, AA_TILE_KEY0(i + 1), tid, sm.idx);
-#endif
+    // tile i+1 goes straight into the other buffer (every wave finished reading it before the last barrier)
+    if (i + 1 < n_tiles)
+      tile_fetch<MODE>(kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(i + 1), tid, sm.idx,
+                       lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes);
 
     AA_STAMP(0)
     // a wave whose rows all lie above this tile (causal) has nothing to do
     const bool wave_active = (MODE == kSparse) || (key0 <= wr0 + 32 * QB - 1);
     if (wave_active) {
-      const __bf16* ks_ = sm.t.k[buf] + k_rd;
+      const char* ks_ = sm.t.k[buf];
       // ---- S^T = K Q^T ------------------------------------------------------------------------
       // K operands are fetched from LDS four k-steps (eight reads) ahead of the MFMAs that use them;
       // the scheduling fences keep that distance (left alone, the reads sink next to their use and
@@ -280,13 +293,13 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) ka[ks][kb] = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * ks);
+        for (int kb = 0; kb < 2; ++kb) ka[ks][kb] = *reinterpret_cast<const bf16x8*>(ks_ + k_rd[ks] + 32 * kb * kRowBytes);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
         if (ks + 4 < 8) {
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) ka[ks + 4][kb] = *reinterpret_cast<const bf16x8*>(ks_ + 32 * kb * kRowStride + 16 * (ks + 4));
+          for (int kb = 0; kb < 2; ++kb) ka[ks + 4][kb] = *reinterpret_cast<const bf16x8*>(ks_ + k_rd[ks + 4] + 32 * kb * kRowBytes);
         }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -371,11 +384,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
           float pv[16];
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-#if defined(AA_ABLATE) && (AA_ABLATE == 2)
-            pv[r] = s[kb][qb][r];
-#else
             pv[r] = fast_exp2(s[kb][qb][r]);
-#endif
             sum += pv[r];
           }
 #pragma unroll
@@ -394,20 +403,20 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
       AA_STAMP(2)
       // ---- O^T += V^T P^T ---------------------------------------------------------------------
       // 16 operand fetches (two transposing reads each), kept four ahead of their MFMAs
-      const __bf16* vs_ = sm.t.v[buf] + v_rd;
+      const char* vs_ = sm.t.v[buf];
       shortx4 vlo[16], vhi[16];
-#define AA_V_SRC(i) (vs_ + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowStride + 32 * ((i) & 3))
+#define AA_V_SRC(i) (vs_ + v_rd[(i) & 3] + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i)));
-        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i) + 8 * kRowStride));
+        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i) + 8 * kRowBytes));
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {  // i = (kb*2 + st)*4 + db
         if (i + 4 < 16) {
           vlo[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4)));
-          vhi[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4) + 8 * kRowStride));
+          vhi[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4) + 8 * kRowBytes));
         }
         typedef short shortx8 __attribute__((ext_vector_type(8)));
         const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -421,11 +430,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
       AA_STAMP(3)
     }
 
-#if defined(AA_ABLATE) && (AA_ABLATE == 3)
-    if (i < 1) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
-#else
-    if (i + 1 < n_tiles) tile_store(tr, sm.t.k[buf ^ 1], sm.t.v[buf ^ 1], tid);
-#endif
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
     __syncthreads();
     AA_STAMP(4)
   }
