@@ -102,27 +102,8 @@ int check_launch(hipError_t e, const char* who) {
   return AA_OK;
 }
 
-// query rows per work-group = 128 * qb; 1 unless AA_FLASH_QB=2 is exported (tuning knob)
-int flash_qb() {
-  static const int qb = [] {
-    const char* e = getenv("AA_FLASH_QB");
-    return (e && e[0] == '2') ? 2 : 1;
-  }();
-  return qb;
-}
-
-// AA_FLASH_PIPE=1 selects the software-pipelined 256-row flash kernels (aa_flash2.hip) instead of the
-// default 128-row ones (aa_flash.hip); same results, kept selectable for measurements
-bool flash_pipelined() {
-  static const bool on = [] {
-    const char* e = getenv("AA_FLASH_PIPE");
-    return e && e[0] == '1';
-  }();
-  return on;
-}
-
 hipError_t run_flash(const FlashArgs& a, int mode, hipStream_t stream) {
-  return flash_pipelined() ? launch_flash2(a, mode, stream) : launch_flash(a, mode, flash_qb(), stream);
+  return launch_flash(a, mode, stream);
 }
 
 size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
@@ -341,8 +322,8 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                         float sm_scale, void* stream) {
   const char* who = "aa_dense_causal_fwd";
   int rc;
-  if (n_ctx <= 0 || n_ctx % 256 != 0) {
-    set_error("%s: n_ctx %d must be a positive multiple of 256", who, n_ctx);
+  if (n_ctx <= 0 || n_ctx % 128 != 0) {
+    set_error("%s: n_ctx %d must be a positive multiple of 128", who, n_ctx);
     return AA_EUNSUPPORTED;
   }
   Dims d = {batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16};

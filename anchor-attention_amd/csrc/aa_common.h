@@ -36,6 +36,14 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // value held by the lane 32 positions away (the two halves of a wave share MFMA columns)
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// max of a value and its counterpart 32 lanes away, without a trip through LDS: v_permlane32_swap hands every
+// lane the lower half's value (result 0) and the upper half's value (result 1)
+__device__ __forceinline__ float max_with_other_half(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // ---- geometry --------------------------------------------------------------------------------
 // Index lists are packed per (batch, query head): big block bb can select at most
 // cap(bb) = bb*S - 2*bs keys (candidates are [bs, bb*S - bs)), and its list starts at

@@ -3,7 +3,7 @@
 //   kSparse : stage 3 - resumes from (M, L, Acc) over K/V rows gathered at selected indices
 //   kDense  : plain causal attention (baseline)
 //
-// Formulation.  A wave owns 32*QB query rows and computes the TRANSPOSED score tile
+// Formulation.  A wave owns 32 query rows and computes the TRANSPOSED score tile
 //   S^T[key][query] = K[key][:] . Q[query][:]      (MFMA A = K rows from LDS, B = Q from registers)
 // so that in the 32x32 accumulator layout a lane holds one query column: the soft-max statistics
 // of a query are then plain per-lane scalars (one exchange with the lane 32 positions away
@@ -22,7 +22,11 @@
 // after the first tiles) does the wave take a slow path that shifts the tile, re-bases the tuple and
 // rescales the accumulators - which is exact for the lanes whose max did not move (shift 0, factor 1).
 //
-// Work-group = 4 waves = 128*QB query rows; keys are consumed 64 at a time through a
+// Inside a 64-key tile the two 32-key halves are staggered so that matrix and vector work overlap
+// within a wave: S0 | S1 with soft-max(S0) | P0.V0 with soft-max(S1) | P1.V1.  The online soft-max
+// therefore advances 32 keys at a time.
+//
+// Work-group = 4 waves = 128 query rows; keys are consumed 64 at a time through a
 // double-buffered LDS tile that the memory system fills directly (global_load_lds_dwordx4: no staging
 // registers, no LDS store instructions).  Such a load writes lane L's 16 bytes at M0 + 16*L, so LDS rows
 // are unpadded 256 bytes; bank conflicts are avoided by XOR-swizzling the 16-byte chunks of a row, which
@@ -47,17 +51,21 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
 
-template <int QB, bool WITH_IDX>
+template <bool WITH_IDX>
 struct FlashSmem {
   union {
     struct {
       char k[2][kTileBytes];
       char v[2][kTileBytes];
     } t;
-    __bf16 os[4][32 * QB * kOsStride];  // epilogue staging, reuses the tile space
+    __bf16 os[4][32 * kOsStride];  // epilogue staging, reuses the tile space
   };
   int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
+#ifdef AA_ONE_WG
+  char pad_one_wg[24576];
+#endif
 };
 
 __device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale, const bool bf16_chain) {
@@ -88,33 +96,31 @@ __device__ __forceinline__ void load16_to_lds(const char* base, const uint32_t b
 }
 
 // One K/V tile: wave w fills LDS rows 16*j + 4*w .. +3 (j = 0..3), i.e. thread t brings the chunk that belongs in
-// slot (t & 15) of row (t >> 4) + 16*j.  `kb`/`vb` are the wave-uniform head bases, `k_col`/`v_col` the byte
-// offset of this thread's (swizzled) chunk inside a row, `lds_k`/`lds_v` the LDS address of row 4*w of the
-// destination tile.  Gathered tiles take their row numbers from the LDS window of the index list (a dependent
-// global load per tile would put a full memory latency on the critical path of every tile).
+// slot (t & 15) of row (t >> 4) + 16*j; tile_fetch_one issues one of the tile's eight loads.  `kb`/`vb` are the
+// wave-uniform head bases, `k_col`/`v_col` the byte offset of this thread's (swizzled) chunk inside a row,
+// `lds_k`/`lds_v` the LDS address of row 4*w of the destination tile.  Gathered tiles take their row numbers from
+// the LDS window of the index list (a dependent global load per tile would put a full memory latency on the
+// critical path of every tile).
 template <int MODE>
-__device__ __forceinline__ void tile_fetch(const char* kb, const char* vb, const uint32_t k_row_bytes, const uint32_t v_row_bytes,
-                                           const uint32_t k_col, const uint32_t v_col, const int key0, const int tid,
-                                           const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v) {
-  const int row0 = tid >> 4;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int row = row0 + 16 * j;
-    uint32_t key;
-    if (MODE == kSparse) {
-      key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
-    } else {
-      key = (uint32_t)(key0 + row);
-    }
-    load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
-    load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
+__device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, const char* vb, const uint32_t k_row_bytes,
+                                               const uint32_t v_row_bytes, const uint32_t k_col, const uint32_t v_col, const int key0,
+                                               const int tid, const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v) {
+  const int j = n >> 1;  // load n: K (even n) or V (odd n) rows 16*j + ...
+  const int row = (tid >> 4) + 16 * j;
+  uint32_t key;
+  if (MODE == kSparse) {
+    key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
+  } else {
+    key = (uint32_t)(key0 + row);
   }
+  if ((n & 1) == 0) load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
+  else load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
 }
 
-template <int QB, int MODE>
-__global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const FlashArgs p) {
-  __shared__ __attribute__((aligned(16))) FlashSmem<QB, MODE == kSparse> sm;
-  constexpr int BM = 128 * QB;
+template <int MODE>
+__global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
+  __shared__ __attribute__((aligned(16))) FlashSmem<MODE == kSparse> sm;
+  constexpr int BM = 128;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -135,7 +141,8 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   const int R0 = qblk * BM;
   const int S = p.big_block;
   const int bb = R0 / S;
-  const int wr0 = R0 + wave * 32 * QB;
+  const int wr0 = R0 + wave * 32;
+  const int my_row = wr0 + c32;
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 #ifdef AA_CLOCKS  // timing experiments only: shader-clock and 100 MHz reference stamps
 #ifndef AA_CLOCKS_QBLK
@@ -184,69 +191,60 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   const uint32_t k_col = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15)) * 16u;
   const uint32_t v_col = (uint32_t)((tid & 15) ^ (((tid >> 4) & 7) << 1)) * 16u;
   const uint32_t lds_k0 = lds_addr(sm.t.k[0]) + wave * 4 * kRowBytes, lds_v0 = lds_addr(sm.t.v[0]) + wave * 4 * kRowBytes;
-  if (n_tiles > 0) tile_fetch<MODE>(kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0);
+  if (n_tiles > 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0);
+  }
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
-  bf16x8 qreg[QB][8];
+  bf16x8 qreg[8];
   {
     const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
+    const __bf16* row = qp + (int64_t)my_row * p.q_sn + 8 * half;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const __bf16* row = qp + (int64_t)(wr0 + 32 * qb + c32) * p.q_sn + 8 * half;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qreg[qb][ks] = scale_q8(*reinterpret_cast<const u32x4*>(row + 16 * ks), p.sm_scale, chain);
-    }
+    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8(*reinterpret_cast<const u32x4*>(row + 16 * ks), p.sm_scale, chain);
   }
 
   // ---- running state -------------------------------------------------------------------------
-  float m_run[QB], l_run[QB];
-  floatx16 acc[4][QB];
+  float m_run, l_run;
+  floatx16 acc[4];
   if (MODE == kSparse) {
+    m_run = p.M[bh * p.n_ctx + my_row];
+    l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
+    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const int row = wr0 + 32 * qb + c32;
-      m_run[qb] = p.M[bh * p.n_ctx + row];
-      l_run[qb] = half == 0 ? p.L[bh * p.n_ctx + row] : 0.f;  // the two halves are summed at the end
-      const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + row / 32) * 16) * 256 + lane * 4;
+    for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int rg = 0; rg < 4; ++rg) {
+        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
-#pragma unroll
-          for (int c = 0; c < 4; ++c) acc[db][qb][rg * 4 + c] = t[c];
-        }
-    }
+        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
+      }
   } else {
+    m_run = -INFINITY;
+    l_run = 0.f;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      m_run[qb] = -INFINITY;
-      l_run[qb] = 0.f;
+    for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[db][qb][r] = 0.f;
-    }
+      for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
   }
 
   // m_ref is what the score accumulators are pre-loaded with (negated); it equals m_run except before
   // the first tile of a fresh row (m_run = -inf, m_ref = 0)
-  float m_ref[QB];
-  floatx16 negm[QB];
+  float m_ref = (MODE == kSparse) ? m_run : 0.f;
+  floatx16 negm;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    m_ref[qb] = (MODE == kSparse) ? m_run[qb] : 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) negm[qb][r] = -m_ref[qb];
-  }
+  for (int r = 0; r < 16; ++r) negm[r] = -m_ref;
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
   __syncthreads();
 
   // per-lane LDS byte offsets.  K: row c32 (+32*kb), chunk 2*ks + half, swizzled with the row's low four bits.
+  // (absolute LDS addresses into the current buffer; the 32-key half and the row steps are immediate offsets)
   uint32_t k_rd[8];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) k_rd[ks] = c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  for (int ks = 0; ks < 8; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
   // transposing V read i: a group of 16 lanes covers 16 head-dim columns; lane points at row r0 = 4*half + (lane%16)/4
   // (+ multiples of 8, which leave r0 = row & 7 alone), bf16 columns 32*(i&3) + 16*((lane>>4)&1) + 4*(lane&3): chunk
   // 4*(i&3) + y0 with y0 < 4, swizzled with r0 << 1 -> one offset per value of i & 3
@@ -255,7 +253,7 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
     const int r0 = 4 * half + ((lane & 15) >> 2);
     const int y0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) v_rd[m] = r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
+    for (int m = 0; m < 4; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
   }
 
 #ifdef AA_CLOCKS
@@ -265,6 +263,57 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
 #else
 #define AA_STAMP(i)
 #endif
+
+  // key (or list position) that accumulator register r of 32-key half kb of the tile at key0 stands for
+#define AA_KEY_OF(kb, r) (key0 + 32 * (kb) + 8 * ((r) >> 2) + 4 * half + ((r) & 3))
+  // causal / list-end mask of one 32-key half (only tiles on the diagonal or at the end of a list need it)
+#define AA_MASK(sx, kb)                                                              \
+  if (MODE != kSparse) {                                                             \
+    if (key0 + 32 * (kb) + 31 > wr0) {                                               \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r)                                 \
+        if (AA_KEY_OF(kb, r) > my_row) sx[r] = -INFINITY;                            \
+    }                                                                                \
+  } else if (key0 + 32 * (kb) + 32 > cnt) {                                          \
+    _Pragma("unroll") for (int r = 0; r < 16; ++r)                                   \
+      if (AA_KEY_OF(kb, r) >= cnt) sx[r] = -INFINITY;                                \
+  }
+  // row max of one half (both halves of the wave hold the same query), relative to m_ref
+#define AA_ROWMAX(sx, mx)                                                            \
+  {                                                                                  \
+    float t0 = fmaxf(fmaxf(sx[0], sx[1]), sx[2]), t1 = fmaxf(fmaxf(sx[3], sx[4]), sx[5]);      \
+    float t2 = fmaxf(fmaxf(sx[6], sx[7]), sx[8]), t3 = fmaxf(fmaxf(sx[9], sx[10]), sx[11]);    \
+    float t4 = fmaxf(fmaxf(sx[12], sx[13]), sx[14]);                                 \
+    t0 = fmaxf(fmaxf(t0, t1), t2);                                                   \
+    t3 = fmaxf(fmaxf(t3, t4), sx[15]);                                               \
+    t0 = fmaxf(t0, t3);                                                              \
+    mx = max_with_other_half(t0);                                                     \
+  }
+  // p = exp2(s) for accumulator registers 4c .. 4c+3 of one half, summed and rounded into the P^T fragment words
+#define AA_EXP_CHUNK(sx, pw, sum, c)                                                 \
+  {                                                                                  \
+    const float e0 = fast_exp2(sx[4 * (c) + 0]), e1 = fast_exp2(sx[4 * (c) + 1]);    \
+    const float e2 = fast_exp2(sx[4 * (c) + 2]), e3 = fast_exp2(sx[4 * (c) + 3]);    \
+    sum += e0; sum += e1; sum += e2; sum += e3;                                      \
+    pw[(c) >> 1][2 * ((c) & 1) + 0] = pack_bf16(e0, e1);                             \
+    pw[(c) >> 1][2 * ((c) & 1) + 1] = pack_bf16(e2, e3);                             \
+  }
+  // V operand fetch i (two transposing reads): i = (kb*2 + st)*4 + db
+#define AA_V_SRC(i) (v_rd[(i) & 3] + (uint32_t)((32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes))
+#define AA_V_FETCH(i)                                                                                  \
+  {                                                                                                    \
+    vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(AA_V_SRC(i)));                     \
+    vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(AA_V_SRC(i) + 8u * kRowBytes));    \
+  }
+#define AA_PV_MFMA(i, pw)                                                                              \
+  {                                                                                                    \
+    typedef short shortx8 __attribute__((ext_vector_type(8)));                                         \
+    const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);                \
+    acc[(i) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&av),      \
+                                                           *reinterpret_cast<const bf16x8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3], 0, 0, 0); \
+  }
+#define AA_FENCE __builtin_amdgcn_sched_barrier(0)
+
+  int32_t buf_step = kTileBytes;  // what takes the read addresses to the other LDS buffer
   for (int i = 0; i < n_tiles; ++i) {
     const int buf = i & 1;
     AA_STAMP(5)
@@ -274,167 +323,173 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
       fill_index_window((i + 1) * kBN);
       __syncthreads();
     }
-    // tile i+1 goes straight into the other buffer (every wave finished reading it before the last barrier)
-    if (i + 1 < n_tiles)
-      tile_fetch<MODE>(kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(i + 1), tid, sm.idx,
-                       lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes);
+    // Tile i+1 goes straight into the other buffer (every wave finished reading it before the last barrier).  Its
+    // eight load instructions are spread over the first MFMAs of this tile: issued in one burst by all four waves
+    // they queue up behind each other in the memory pipeline and every wave stalls for the length of the queue.
+    // (the last tile fetches itself once more into the idle buffer, which keeps the instruction stream free of branches)
+    const int i_next = i + 1 < n_tiles ? i + 1 : i;
+    const int key0_next = AA_TILE_KEY0(i_next);
+#ifdef AA_NO_FETCH  // timing experiment: tiles after the first are not fetched (results are meaningless)
+#define AA_FETCH_ONE(n)
+#else
+#define AA_FETCH_ONE(n)                                                                                               \
+  tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,   \
+                                  lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes);
+#endif
 
     AA_STAMP(0)
-    // a wave whose rows all lie above this tile (causal) has nothing to do
-    const bool wave_active = (MODE == kSparse) || (key0 <= wr0 + 32 * QB - 1);
-    if (wave_active) {
-      const char* ks_ = sm.t.k[buf];
-      // ---- S^T = K Q^T ------------------------------------------------------------------------
-      // K operands are fetched from LDS four k-steps (eight reads) ahead of the MFMAs that use them;
-      // the scheduling fences keep that distance (left alone, the reads sink next to their use and
-      // every MFMA then waits out a full LDS latency).
-      floatx16 s[2][QB];
-      bf16x8 ka[8][2];
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) ka[ks][kb] = *reinterpret_cast<const bf16x8*>(ks_ + k_rd[ks] + 32 * kb * kRowBytes);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        if (ks + 4 < 8) {
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb) ka[ks + 4][kb] = *reinterpret_cast<const bf16x8*>(ks_ + k_rd[ks + 4] + 32 * kb * kRowBytes);
-        }
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            if (ks == 0) {
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], negm[qb], 0, 0, 0);
-            } else {
-              s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kb], qreg[qb][ks], s[kb][qb], 0, 0, 0);
-            }
-          }
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    // (a wave whose rows all lie above this tile - two of the four waves on the last tile of a causal work-group -
+    // runs it fully masked: it would only wait at the barrier for the others anyway)
+    {
+      floatx16 s0, s1;
+      bf16x8 ka[16];            // K operand t = kb*8 + ks, fetched from LDS four MFMAs ahead of its use
+      shortx4 vlo[16], vhi[16];  // V operands, same distance
+      u32x4 pw0[2], pw1[2];      // P^T fragments (bf16 pairs) of the two halves
+      float mx0, mx1, sum0 = 0.f, sum1 = 0.f, shift0 = 0.f, alpha1 = 1.f;
+#define AA_K_FETCH(t) ka[t] = *(const lds_bf16x8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(32 * ((t) >> 3) * kRowBytes))
 
+      // ---- phase A: S0^T = K0 Q^T -------------------------------------------------------------
+      // (the scheduling fences keep the operand fetches at their distance: left alone, the reads sink next
+      // to their use and every MFMA then waits out a full LDS latency)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) AA_K_FETCH(t);
+      AA_FENCE;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        AA_K_FETCH(t + 4);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[t], qreg[t], t == 0 ? negm : s0, 0, 0, 0);
+        AA_FETCH_ONE(t)
+        AA_FENCE;
+      }
       AA_STAMP(1)
-      // ---- masks ------------------------------------------------------------------------------
-      if (MODE != kSparse) {
-        if (key0 + kBN - 1 > wr0) {  // tile touches the diagonal of this wave
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (key > wr0 + 32 * qb + c32) s[kb][qb][r] = -INFINITY;
-              }
-        }
-      } else if (key0 + kBN > cnt) {  // last, partly filled chunk of the index list
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int pos = key0 + 32 * kb + 8 * (r >> 2) + 4 * half + (r & 3);
-              if (pos >= cnt) s[kb][qb][r] = -INFINITY;
-            }
-      }
 
-      // ---- online soft-max (exp2 domain); s holds S - m_ref ---------------------------------------
-      bf16x8 pfrag[2][QB][2];
-      float mxr[QB];
-      bool moved = false;
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        float mx = s[0][qb][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kb][qb][r]);
-        mxr[qb] = fmaxf(mx, xor32(mx));
-        moved |= (m_ref[qb] + mxr[qb] > m_run[qb]);
-      }
-      if (__any(moved)) {
+      // ---- phase B: S1^T = K1 Q^T, with the soft-max of S0 between the MFMAs ---------------------
+      AA_K_FETCH(12);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[8], qreg[0], negm, 0, 0, 0);
+      AA_FENCE;
+      AA_K_FETCH(13);
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[9], qreg[1], s1, 0, 0, 0);
+      AA_FENCE;
+      AA_MASK(s0, 0)
+      AA_ROWMAX(s0, mx0)
+      const bool moved0 = __any(m_ref + mx0 > m_run);
+      if (moved0) {
         // slow path: some row's max grew.  Lanes whose max did not move get shift 0 and alpha 1 (exact).
+        // S1 is being accumulated on top of the old -m_ref and is shifted once it is complete.
+        const float m_new = fmaxf(m_run, m_ref + mx0);
+        const float alpha = fast_exp2(m_run - m_new);
+        shift0 = m_new - m_ref;
+        m_run = m_new;
+        m_ref = m_new;
+        l_run *= alpha;
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          const float m_new = fmaxf(m_run[qb], m_ref[qb] + mxr[qb]);
-          const float alpha = fast_exp2(m_run[qb] - m_new);
-          const float shift = m_new - m_ref[qb];
-          m_run[qb] = m_new;
-          m_ref[qb] = m_new;
-          l_run[qb] *= alpha;
+        for (int r = 0; r < 16; ++r) s0[r] -= shift0;
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
+        for (int r = 0; r < 16; ++r) negm[r] = -m_new;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[kb][qb][r] -= shift;
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) negm[qb][r] = -m_new;
-#pragma unroll
-          for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[db][qb][r] *= alpha;
-        }
+          for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
       }
+      AA_FENCE;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        float sum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          float pv[16];
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            pv[r] = fast_exp2(s[kb][qb][r]);
-            sum += pv[r];
-          }
-#pragma unroll
-          for (int st = 0; st < 2; ++st) {
-            u32x4 w;
-            w[0] = pack_bf16(pv[8 * st + 0], pv[8 * st + 1]);
-            w[1] = pack_bf16(pv[8 * st + 2], pv[8 * st + 3]);
-            w[2] = pack_bf16(pv[8 * st + 4], pv[8 * st + 5]);
-            w[3] = pack_bf16(pv[8 * st + 6], pv[8 * st + 7]);
-            pfrag[kb][qb][st] = *reinterpret_cast<bf16x8*>(&w);
-          }
-        }
-        l_run[qb] += sum;
+      for (int c = 0; c < 4; ++c) {
+        if (c < 2) AA_K_FETCH(14 + c);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[10 + c], qreg[2 + c], s1, 0, 0, 0);
+        AA_EXP_CHUNK(s0, pw0, sum0, c)
+        AA_FENCE;
       }
-
+      l_run += sum0;
+      AA_V_FETCH(0)
+      AA_V_FETCH(1)
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[14], qreg[6], s1, 0, 0, 0);
+      AA_FENCE;
+      AA_V_FETCH(2)
+      AA_V_FETCH(3)
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[15], qreg[7], s1, 0, 0, 0);
+      AA_FENCE;
       AA_STAMP(2)
-      // ---- O^T += V^T P^T ---------------------------------------------------------------------
-      // 16 operand fetches (two transposing reads each), kept four ahead of their MFMAs
-      const char* vs_ = sm.t.v[buf];
-      shortx4 vlo[16], vhi[16];
-#define AA_V_SRC(i) (vs_ + v_rd[(i) & 3] + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i)));
-        vhi[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i) + 8 * kRowBytes));
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {  // i = (kb*2 + st)*4 + db
-        if (i + 4 < 16) {
-          vlo[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4)));
-          vhi[i + 4] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(AA_V_SRC(i + 4) + 8 * kRowBytes));
-        }
-        typedef short shortx8 __attribute__((ext_vector_type(8)));
-        const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&av);
-        const int kb = i >> 3, st = (i >> 2) & 1, db = i & 3;
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) acc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[kb][qb][st], acc[db][qb], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#undef AA_V_SRC
-      AA_STAMP(3)
-    }
 
+      // ---- phase C: O^T += V0^T P0^T, with the soft-max of S1 between the MFMAs --------------------
+      AA_V_FETCH(4)
+      AA_PV_MFMA(0, pw0)
+      AA_FENCE;
+      AA_V_FETCH(5)
+      AA_PV_MFMA(1, pw0)
+      AA_FENCE;
+      if (moved0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s1[r] -= shift0;
+      }
+      AA_MASK(s1, 1)
+      AA_ROWMAX(s1, mx1)
+      const bool moved1 = __any(m_ref + mx1 > m_run);
+      if (moved1) {
+        // as above, except that O^T is rescaled only after the P0 V0 products in flight have been added
+        const float m_new = fmaxf(m_run, m_ref + mx1);
+        alpha1 = fast_exp2(m_run - m_new);
+        const float shift = m_new - m_ref;
+        m_run = m_new;
+        m_ref = m_new;
+        l_run *= alpha1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s1[r] -= shift;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) negm[r] = -m_new;
+      }
+      AA_FENCE;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        AA_V_FETCH(6 + c)
+        AA_PV_MFMA(2 + c, pw0)
+        AA_EXP_CHUNK(s1, pw1, sum1, c)
+        AA_FENCE;
+      }
+      l_run += sum1;
+      AA_V_FETCH(10)
+      AA_PV_MFMA(6, pw0)
+      AA_FENCE;
+      AA_V_FETCH(11)
+      AA_PV_MFMA(7, pw0)
+      AA_FENCE;
+      if (moved1) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[db][r] *= alpha1;
+      }
+
+      // ---- phase D: O^T += V1^T P1^T ---------------------------------------------------------------
+#pragma unroll
+      for (int j = 8; j < 16; ++j) {
+        if (j + 4 < 16) AA_V_FETCH(j + 4)
+        AA_PV_MFMA(j, pw1)
+        AA_FENCE;
+      }
+      AA_STAMP(3)
+#undef AA_K_FETCH
+    }
+#undef AA_FETCH_ONE
+
+    // the read addresses follow the tiles into the other buffer
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_rd[ks] += buf_step;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) v_rd[m] += buf_step;
+    buf_step = -buf_step;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
     __syncthreads();
     AA_STAMP(4)
   }
 #undef AA_TILE_KEY0
+#undef AA_KEY_OF
+#undef AA_MASK
+#undef AA_ROWMAX
+#undef AA_EXP_CHUNK
+#undef AA_V_SRC
+#undef AA_V_FETCH
+#undef AA_PV_MFMA
+#undef AA_FENCE
 
 #ifdef AA_CLOCKS
   if (MODE != kDense && tid == 0 && qblk == AA_CLOCKS_QBLK && hq == 0 && b == 0) {
@@ -445,47 +500,39 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   }
 #endif
   // ---- epilogue --------------------------------------------------------------------------------
+  const float l_tot = l_run + xor32(l_run);
   if (MODE == kAnchor) {
+    if (half == 0) {
+      p.M_out[bh * p.n_ctx + my_row] = m_run;
+      p.L_out[bh * p.n_ctx + my_row] = l_tot;
+    }
+    float* af = p.acc_out + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const int row = wr0 + 32 * qb + c32;
-      const float l_tot = l_run[qb] + xor32(l_run[qb]);
-      if (half == 0) {
-        p.M_out[bh * p.n_ctx + row] = m_run[qb];
-        p.L_out[bh * p.n_ctx + row] = l_tot;
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        floatx4 t;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) t[c] = acc[db][rg * 4 + c];
+        *reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256) = t;
       }
-      float* af = p.acc_out + ((bh * (p.n_ctx / 32) + row / 32) * 16) * 256 + lane * 4;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          floatx4 t;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) t[c] = acc[db][qb][rg * 4 + c];
-          *reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256) = t;
-        }
-    }
   } else {
-    // out = bf16(acc / l): stage the wave's [32*QB][128] tile in LDS, then write whole rows
+    // out = bf16(acc / l): stage the wave's [32][128] tile in LDS, then write whole rows
     __bf16* os = sm.os[wave];
+    const float inv = 1.0f / l_tot;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const float l_tot = l_run[qb] + xor32(l_run[qb]);
-      const float inv = 1.0f / l_tot;
+    for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          u32x2 w;
-          w[0] = pack_bf16(acc[db][qb][rg * 4 + 0] * inv, acc[db][qb][rg * 4 + 1] * inv);
-          w[1] = pack_bf16(acc[db][qb][rg * 4 + 2] * inv, acc[db][qb][rg * 4 + 3] * inv);
-          *reinterpret_cast<u32x2*>(&os[(32 * qb + c32) * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
-        }
-    }
+      for (int rg = 0; rg < 4; ++rg) {
+        u32x2 w;
+        w[0] = pack_bf16(acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv);
+        w[1] = pack_bf16(acc[db][rg * 4 + 2] * inv, acc[db][rg * 4 + 3] * inv);
+        *reinterpret_cast<u32x2*>(&os[c32 * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
+      }
     __syncthreads();
     __bf16* op = p.out + b * p.o_sb + hq * p.o_sh;
 #pragma unroll
-    for (int it = 0; it < 8 * QB; ++it) {
+    for (int it = 0; it < 8; ++it) {
       const int r = it * 4 + (lane >> 4), c = lane & 15;
       const u32x4 w = *reinterpret_cast<const u32x4*>(&os[r * kOsStride + 8 * c]);
       *reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c) = w;
@@ -493,23 +540,17 @@ __global__ void __launch_bounds__(256, QB == 1 ? 2 : 1) flash_kernel(const Flash
   }
 }
 
-template <int QB, int MODE>
+template <int MODE>
 static hipError_t launch(const FlashArgs& a, hipStream_t stream) {
-  const int BM = 128 * QB;
-  const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / BM);
-  hipLaunchKernelGGL((flash_kernel<QB, MODE>), dim3(grid), dim3(256), 0, stream, a);
+  const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / 128);
+  hipLaunchKernelGGL((flash_kernel<MODE>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 
-hipError_t launch_flash(const FlashArgs& a, int mode, int qb, hipStream_t stream) {
-  if (qb == 1) {
-    if (mode == kAnchor) return launch<1, kAnchor>(a, stream);
-    if (mode == kSparse) return launch<1, kSparse>(a, stream);
-    return launch<1, kDense>(a, stream);
-  }
-  if (mode == kAnchor) return launch<2, kAnchor>(a, stream);
-  if (mode == kSparse) return launch<2, kSparse>(a, stream);
-  return launch<2, kDense>(a, stream);
+hipError_t launch_flash(const FlashArgs& a, int mode, hipStream_t stream) {
+  if (mode == kAnchor) return launch<kAnchor>(a, stream);
+  if (mode == kSparse) return launch<kSparse>(a, stream);
+  return launch<kDense>(a, stream);
 }
 
 }  // namespace aa

@@ -17,10 +17,8 @@ struct FlashArgs {
   float sm_scale; int scale_mode;
 };
 
-// mode: 0 anchor (stage 1), 1 sparse (stage 3), 2 dense causal.  qb: 32-row query blocks per wave (1|2).
-hipError_t launch_flash(const FlashArgs& a, int mode, int qb, hipStream_t stream);
-// software-pipelined variant, 256-row work-groups (n_ctx % 256 == 0)
-hipError_t launch_flash2(const FlashArgs& a, int mode, hipStream_t stream);
+// mode: 0 anchor (stage 1), 1 sparse (stage 3), 2 dense causal
+hipError_t launch_flash(const FlashArgs& a, int mode, hipStream_t stream);
 
 struct PoolArgs {
   const __bf16* q; int64_t q_sb, q_sh, q_sn;

@@ -128,7 +128,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
 /* ---- dense causal baseline on the same MFMA core --------------------------------------------
  * Counterpart of the reference's dense comparison path (flash_attn_triton.py:83-211, GQA mapping
  * :129-132): plain causal softmax attention, out = bf16(softmax(q k^T * sm_scale) v).
- * n_ctx must be a multiple of 256. */
+ * n_ctx must be a multiple of 128. */
 int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,

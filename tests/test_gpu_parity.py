@@ -44,7 +44,7 @@ def llama_small(mods):
     return (q.cuda(), k.cuda(), v.cuda()), (Q, K, V), res
 
 
-def _packed_lists(hip, coords, counts, N):
+def _packed_lists(hip, coords, counts, N, step=STEP):
     coords = coords.cpu().numpy()
     counts = counts.cpu().numpy().reshape(coords.shape[0], coords.shape[1], -1)
     lib = hip.lib()
@@ -54,15 +54,16 @@ def _packed_lists(hip, coords, counts, N):
         for h in range(coords.shape[1]):
             ph = []
             for bb in range(counts.shape[2]):
-                off = lib.aa_coords_offset(bb, BS, STEP)
+                off = lib.aa_coords_offset(bb, BS, step)
                 ph.append(coords[b, h, off:off + counts[b, h, bb]].copy())
             pb.append(ph)
         out.append(pb)
     return out, counts
 
 
-def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused):
+def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP):
     """Sets equal except excused keys (flip distance < BAND); returns number of excused keys."""
+    S = BS * step
     B, Hq = got_counts.shape[:2]
     group = Hq // K.shape[1]
     excused = 0
@@ -80,7 +81,7 @@ def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused)
                 if qbar is None:
                     qbar = ao.pooled_queries(Q[b, h], BS)
                     abar, mean = ao.pooled_anchors(M[b, h], BS)
-                rows = slice(bb * STEP, (bb + 1) * STEP)
+                rows = slice(bb * step, (bb + 1) * step)
                 for j in sym:
                     d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta)
                     assert d < BAND, f"key {j} (b={b},h={h},bb={bb}) differs and is {d:.4g} from any decision flip"
@@ -175,21 +176,21 @@ def test_stage3_matches_oracle_given_same_state(mods, llama_small):
 
 
 # ------------------------------------------------------------------------------------ whole operator
-def _end_to_end(mods, q, k, v, theta, max_excused=6, rope_note=""):
+def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP):
     hip, v4, st, ao = mods
     Q, K, V = _np(q, k, v)
-    res = ao.anchor_attn_reference(Q, K, V, difference=theta)
+    res = ao.anchor_attn_reference(Q, K, V, step=step, difference=theta)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
-    out, ratio = v4.anchor_attn(qd, kd, vd, difference=theta)
+    out, ratio = v4.anchor_attn(qd, kd, vd, step=step, difference=theta)
     B, H, N, _ = q.shape
     # stage outputs for index parity come from the staged entry points on the same inputs
-    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
-    coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, theta * LOG2E, B, H, N, D, SM)
-    got, got_counts = _packed_lists(hip, coords, counts, N)
-    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused)
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, step, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(qd, kd, M, BS, step, theta * LOG2E, B, H, N, D, SM)
+    got, got_counts = _packed_lists(hip, coords, counts, N, step)
+    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step)
     err = np.abs(out.float().cpu().numpy() - res.out)
     assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
-    want_ratio = got_counts.sum() / ((B * H * N * N / (BS * STEP)) // 2)
+    want_ratio = got_counts.sum() / ((B * H * N * N / (BS * step)) // 2)
     assert abs(float(ratio) - want_ratio) < 1e-6
     return res, out
 
@@ -219,6 +220,36 @@ def test_anchor_attn_dense_regime_literal_qbar(mods):
     q, k, v, _ = _case(3 * S, 2, 1, 32, seed=4, qbar_mode="literal")
     res, _ = _end_to_end(mods, q, k, v, 12.0, max_excused=50)
     assert res.counts[0, 0, 2] > 3000
+
+
+def test_anchor_attn_step_32(mods):
+    """step = 32: 4096-key big blocks, 32 pooled rows per big block (one item per stage-2 MFMA)."""
+    q, k, v, _ = _case(3 * 4096, 4, 2, 96, seed=41)
+    res, _ = _end_to_end(mods, q, k, v, 12.0, step=32)
+    assert res.counts.sum() > 0 and res.counts[:, :, 0].sum() == 0
+
+
+def test_anchor_attn_batch_of_two(mods):
+    """Two different sequences in one call: every (batch, head) pair is independent."""
+    a = _case(2 * S, 4, 2, 48, seed=51)
+    b = _case(2 * S, 4, 2, 48, seed=52)
+    q, k, v = (torch.cat([x, y], 0) for x, y in zip(a[:3], b[:3]))
+    res, out = _end_to_end(mods, q, k, v, 12.0)
+    hip, v4, st, ao = mods
+    single = v4.anchor_attn(b[0].cuda(), b[1].cuda(), b[2].cuda(), return_computational_ratio=False)
+    assert torch.equal(out[1:].cpu(), single.cpu())
+
+
+def test_single_big_block_is_plain_causal_attention(mods):
+    """N = S: no candidates exist, nothing is selected, the output is causal attention."""
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(S, 4, 1, 16, seed=61)
+    out, ratio = v4.anchor_attn(q.cuda(), k.cuda(), v.cuda())
+    assert float(ratio) == 0.0
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(4, 1), v.double().repeat_interleave(4, 1), is_causal=True)
+    err = (out.cpu().double() - ref).abs()
+    assert err.max() < 3e-2 and err.mean() < 2e-3
 
 
 def test_theta_minus_inf_two_big_blocks_equals_library_attention(mods):
@@ -300,3 +331,80 @@ def test_constant_values_at_32k(mods):
     assert 0 < float(ratio) < 0.2
     err = (out.float().cpu() - row.float()).abs()
     assert err.max() <= 2e-2
+
+
+def test_full_size_128k_sampled_parity(mods):
+    """BASELINE config 2 (Llama-3.1-8B layer, 128k tokens, 32/8 heads) through all three stages; sampled
+    rows and sampled (head, big block) pairs are recomputed on the host in float64 / with the oracle's
+    stage-2 arithmetic and compared to the same tolerances as the small cases."""
+    hip, v4, st, ao = mods
+    from bench import make_inputs
+    q, k, v = make_inputs("config2_llama8b_128k", 0, "shared", "cuda:0")
+    B, H, N, _ = q.shape
+    Hkv, group, theta = k.shape[1], q.shape[1] // k.shape[1], 12.0
+    L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(q, k, M, BS, STEP, theta * LOG2E, B, H, N, D, SM)
+    out = v4._stage3(q, k, v, coords, counts, L, M, Acc, SM, BS, STEP)
+    fused, ratio = v4.anchor_attn(q, k, v, difference=theta)
+    assert torch.equal(out, fused)  # one-call entry point == staged entry points, bit for bit
+    assert 0.001 < float(ratio) < 0.05
+    lib = hip.lib()
+    cnt = counts.reshape(B, H, N // S).cpu().numpy()
+    per_head = lib.aa_coords_entries_per_head(N, BS, STEP)
+
+    def index_list(h, bb):
+        off = lib.aa_coords_offset(bb, BS, STEP)
+        return coords.reshape(B, H, per_head)[0, h, off:off + int(cnt[0, h, bb])].cpu().numpy()
+
+    rng = np.random.default_rng(3)
+    # ---- stage 2 on sampled (head, big block) pairs, the last big block included
+    for h, bb in [(0, N // S - 1), (13, 17), (31, 1), (22, 40)]:
+        rows = slice(bb * S, (bb + 1) * S)
+        Qb = q[0, h, rows].float().cpu().numpy()
+        Mb = M[0, h, rows].cpu().numpy()
+        Kc = k[0, h // group, BS:bb * S - BS].float().cpu().numpy()
+        qbar = ao.pooled_queries(Qb, BS)
+        abar, mean = ao.pooled_anchors(Mb, BS)
+        sc, _ = ao.stage2_scores(qbar, Kc, SM)
+        want = (np.nonzero(((sc + np.float32(theta * LOG2E)) >= abar[:, None]).any(axis=0))[0] + BS).astype(np.int32)
+        got = index_list(h, bb)
+        assert np.all(np.diff(got) > 0)
+        for j in np.setxor1d(got, want):
+            d_ = ao.stage2_flip_distance(qbar, abar, mean, k[0, h // group, int(j)].float().cpu().numpy(), SM, theta)
+            assert d_ < BAND, (h, bb, int(j), d_)
+        assert np.setxor1d(got, want).size <= 3
+    # ---- stages 1 and 3 on sampled rows (float64 on the host; P rounded to bf16 as the kernels do)
+    out_rows = []
+    for h, r in [(0, 0), (0, N - 1), (5, 2047), (9, 2048), (17, 70000), (31, N - 2048), (26, int(rng.integers(S, N)))]:
+        bb = r // S
+        kv = h // group
+        keys1 = np.unique(np.concatenate([np.arange(0, min(S, r + 1)), np.arange(bb * S, r + 1)]))
+        K1 = k[0, kv, keys1].double().cpu().numpy()
+        V1 = v[0, kv, keys1].double().cpu().numpy()
+        qrow = q[0, h, r].float().cpu().numpy()
+        q1 = ao.q1_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        s1 = K1 @ q1
+        m1 = s1.max()
+        p1 = np.exp2(s1 - m1)
+        l1 = p1.sum()
+        a1 = ao.rn16(p1.astype(np.float32)).astype(np.float64) @ V1
+        assert abs(float(M[0, h, r]) - m1) < 3e-4
+        assert abs(float(L[0, h, r]) - l1) / l1 < 1e-3
+        lst = index_list(h, bb)
+        q3 = ao.q3_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        if lst.size:
+            K3 = k[0, kv, lst].double().cpu().numpy()
+            V3 = v[0, kv, lst].double().cpu().numpy()
+            s3 = K3 @ q3
+            m = max(m1, s3.max())
+            p3 = np.exp2(s3 - m)
+            num = a1 * np.exp2(m1 - m) + ao.rn16(p3.astype(np.float32)).astype(np.float64) @ V3
+            den = l1 * np.exp2(m1 - m) + p3.sum()
+        else:
+            num, den = a1, l1
+        want_row = num / den
+        got_row = out[0, h, r].double().cpu().numpy()
+        err = np.abs(got_row - want_row)
+        assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (h, r, err.max(), err.mean())
+        out_rows.append(err.max())
+    assert len(out_rows) == 7
