@@ -1,0 +1,93 @@
+"""End-to-end prefill of a Llama-architecture model whose attention is the AnchorAttention operator.
+
+BASELINE config 4: the 32-layer Llama-3.1-8B architecture (hidden 4096, FFN 14336, 32/8 heads, vocab 128256,
+RoPE base 5e5) with random-init bf16 weights and random token ids at N = 131072 on one GPU; reports the
+prefill time with the operator, its attention share, and the same model on the library's dense attention.
+There is no checkpoint or dataset involved: weights and tokens are synthetic, so the sparsity a trained
+model would show is not reproduced - the numbers are timings of the code path, and say so.
+
+    python bench_model_prefill.py                       # config 4
+    python bench_model_prefill.py --layers 2 --n-ctx 8192   # quick check
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--n-ctx", type=int, default=131072)
+    ap.add_argument("--theta", type=float, default=12.0)
+    ap.add_argument("--reps", type=int, default=2)
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention run of the same model")
+    args = ap.parse_args()
+
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from anchor_attn import patch_model
+    from anchor_attn.src.modules.llama import anchor_attention as plug
+
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=args.layers, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=args.n_ctx,
+                      rope_theta=5e5, tie_word_embeddings=False)
+    t0 = time.time()
+    with torch.device(dev):
+        model = LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    print(f"# model built in {time.time() - t0:.1f} s: {sum(p.numel() for p in model.parameters()) / 1e9:.2f} G parameters", file=sys.stderr, flush=True)
+    tokens = torch.randint(0, cfg.vocab_size, (1, args.n_ctx), device=dev)
+
+    # time spent inside the attention plug, by events around every call
+    spans = []
+    inner = plug.anchor_attention_forward
+
+    def timed(*a, **k):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        r = inner(*a, **k)
+        e1.record()
+        spans.append((e0, e1, plug.last_ratio))
+        return r
+
+    def prefill(reps):
+        best = None
+        for _ in range(reps + 1):  # first pass is the warm-up
+            spans.clear()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            with torch.no_grad():
+                out = model(tokens, use_cache=False, logits_to_keep=1).logits
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            attn = sum(a.elapsed_time(b) for a, b, _ in spans)
+            if best is None or ms < best[0]:
+                best = (ms, attn, [float(r) for _, _, r in spans if r is not None], out)
+        return best
+
+    patch_model(model, "anchor_attn", {"theta": args.theta})
+    from transformers import AttentionInterface
+    AttentionInterface.register(plug.ATTN_NAME, timed)
+    ms, attn_ms, ratios, logits = prefill(args.reps)
+    res = {"workload": f"llama3.1-8b architecture, {args.layers} layers, random-init bf16, N={args.n_ctx}, theta={args.theta}",
+           "prefill_ms_anchor_attn": ms, "attention_ms": attn_ms, "attention_share": attn_ms / ms,
+           "mean_sparsity_ratio": sum(ratios) / max(len(ratios), 1), "logits_finite": bool(torch.isfinite(logits).all())}
+    AttentionInterface.register(plug.ATTN_NAME, inner)
+    if not args.no_dense:
+        patch_model(model, "flash")
+        dms, _, _, _ = prefill(1)
+        res["prefill_ms_dense_sdpa"] = dms
+        res["speedup_vs_dense"] = dms / ms
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,113 @@
+"""patch_model and the Hugging Face attention plug: host logic on the CPU (dense branches only - the
+sparse branch needs the GPU and is covered by the gpu-marked tests below)."""
+import types
+
+import pytest
+import torch
+
+
+def _tiny(n_layers=2, **kw):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=n_layers, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=128, vocab_size=1000, max_position_embeddings=16384,
+                      rope_theta=5e5, **kw)
+    return LlamaForCausalLM(cfg).eval()
+
+
+def test_patch_model_validation_and_config():
+    from anchor_attn import get_config_example, patch_model
+    assert get_config_example("anchor_attn") == {"block_size_M": 128, "theta": 12, "step": 16}
+    m = _tiny(1)
+    before = m.config._attn_implementation
+    assert patch_model(m, "default") is m and m.config._attn_implementation == before
+    with pytest.raises(ValueError):
+        patch_model(m, "streaming_llm")  # competitor patterns are not part of this package
+    with pytest.raises(ValueError):
+        patch_model(torch.nn.Linear(2, 2), "anchor_attn")
+    with pytest.raises(ValueError):
+        patch_model(m, "anchor_attn", {"step": 8})
+    patch_model(m, "anchor_attn", {"theta": 11})
+    assert m.config._attn_implementation == "anchor_attn"
+    assert (m.config.block_size_M, m.config.step, m.config.theta) == (128, 16, 11)
+    patch_model(m, "flash")
+    assert m.config._attn_implementation == "sdpa"
+
+
+def test_short_prefill_and_decode_take_the_dense_branch():
+    """Below one big block, and for single-token decode steps against a cache, the plug is dense attention:
+    a patched model generates exactly what the unpatched one does."""
+    from anchor_attn import patch_model
+    ref = _tiny()
+    m = _tiny()
+    m.load_state_dict(ref.state_dict())
+    patch_model(m, "anchor_attn")
+    x = torch.randint(0, 1000, (2, 300))
+    with torch.no_grad():
+        a = ref(x).logits
+        b = m(x).logits
+        assert torch.allclose(a, b, atol=1e-5)
+        ga = ref.generate(x, max_new_tokens=4, do_sample=False)
+        gb = m.generate(x, max_new_tokens=4, do_sample=False)
+    assert torch.equal(ga, gb)
+
+
+def test_plug_dense_branch_matches_reference_math():
+    """Direct call of the plug with a cache-style shape (fewer queries than keys): bottom-right causal."""
+    from anchor_attn.src.modules.llama.anchor_attention import anchor_attention_forward
+    mod = types.SimpleNamespace(config=types.SimpleNamespace(block_size_M=128, step=16, theta=12.0))
+    torch.manual_seed(1)
+    q, k, v = torch.randn(1, 4, 5, 128), torch.randn(1, 2, 37, 128), torch.randn(1, 2, 37, 128)
+    out, w = anchor_attention_forward(mod, q, k, v, None, scaling=0.1)
+    assert w is None and out.shape == (1, 5, 4, 128)
+    kk, vv = k.repeat_interleave(2, 1), v.repeat_interleave(2, 1)
+    s = (q @ kk.transpose(-1, -2)) * 0.1
+    rows = torch.arange(5)[:, None] + 32
+    s = s.masked_fill(torch.arange(37)[None, :] > rows, float("-inf"))
+    want = (s.softmax(-1) @ vv).transpose(1, 2)
+    assert torch.allclose(out, want, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------ GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_tokens", [2 * 2048 + 300, 2 * 2048])
+def test_plug_sparse_branch_is_the_operator_plus_dense_tail(n_tokens):
+    """The plug on HF-layout (transposed, non-contiguous) tensors = anchor_attn on contiguous copies for the
+    rows the operator covers (bit for bit) + dense attention for the tail rows; pad == 0 included."""
+    from anchor_attn.src.modules.llama import anchor_attention as aa
+    from anchor_attn.src.ops.anchor_attn_v4 import anchor_attn
+    from anchor_attn.synthetic import make_qkv
+    q, k, v, _ = make_qkv(n_tokens - n_tokens % 128 + 128 if n_tokens % 128 else n_tokens, 4, 2, n_stripes=64, seed=3)
+    q, k, v = (t[:, :, :n_tokens].cuda() for t in (q, k, v))
+    # what LlamaAttention hands over: [B,H,N,D] views of [B,N,H,D] storage
+    qh, kh, vh = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+    mod = types.SimpleNamespace(config=types.SimpleNamespace(block_size_M=128, step=16, theta=12.0))
+    out, _ = aa.anchor_attention_forward(mod, qh, kh, vh, None, scaling=128 ** -0.5)
+    assert out.shape == (1, n_tokens, 4, 128) and out.is_contiguous()
+    main = n_tokens - n_tokens % 2048
+    want, ratio = anchor_attn(q[:, :, :main].contiguous(), k[:, :, :main].contiguous(), v[:, :, :main].contiguous())
+    assert torch.equal(out.transpose(1, 2)[:, :, :main], want)
+    assert float(aa.last_ratio) == float(ratio) and float(ratio) > 0
+    if n_tokens > main:
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+        err = (out.transpose(1, 2)[:, :, main:].double() - ref[:, :, main:]).abs()
+        assert err.max() < 2e-2
+
+
+@pytest.mark.gpu
+def test_patched_model_equals_dense_model_when_the_window_covers_everything():
+    """theta -> -inf selects nothing; with two big blocks the stage-1 window [0,S) U [bb*S, r] is the whole causal
+    prefix, so a patched model must reproduce the dense (SDPA) model's logits - prefill with a ragged tail."""
+    from anchor_attn import patch_model
+    ref = _tiny().to(torch.bfloat16).cuda()
+    m = _tiny().to(torch.bfloat16).cuda()
+    m.load_state_dict(ref.state_dict())
+    patch_model(m, "anchor_attn", {"theta": -1e4})
+    x = torch.randint(0, 1000, (1, 2 * 2048 + 77), device="cuda")
+    with torch.no_grad():
+        a = ref(x, logits_to_keep=64).logits.float()
+        b = m(x, logits_to_keep=64).logits.float()
+    assert torch.isfinite(b).all()
+    assert (a - b).abs().max() < 0.08 * a.abs().max()
+    assert (a - b).abs().mean() < 0.01 * a.abs().mean() + 1e-3
