@@ -43,6 +43,10 @@ constexpr int kBN = 64;        // keys per LDS tile
 constexpr int kRowBytes = 256;   // one K/V row in LDS (128 bf16, unpadded, chunks swizzled)
 constexpr int kTileBytes = kBN * kRowBytes;
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
+#ifndef AA_DIST
+#define AA_DIST 4
+#endif
+constexpr int kDist = AA_DIST;    // MFMA operands are fetched from LDS this many MFMAs ahead of their use
 constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
@@ -342,34 +346,45 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // runs it fully masked: it would only wait at the barrier for the others anyway)
     {
       floatx16 s0, s1;
-      bf16x8 ka[16];            // K operand t = kb*8 + ks, fetched from LDS four MFMAs ahead of its use
-      shortx4 vlo[16], vhi[16];  // V operands, same distance
+      bf16x8 ka[16];            // K operand of slot n = kb*8 + ks
+      shortx4 vlo[16], vhi[16];  // V operand of slot 16 + i, i = (kb*2 + st)*4 + db
       u32x4 pw0[2], pw1[2];      // P^T fragments (bf16 pairs) of the two halves
       float mx0, mx1, sum0 = 0.f, sum1 = 0.f, shift0 = 0.f, alpha1 = 1.f;
 #define AA_K_FETCH(t) ka[t] = *(const lds_bf16x8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(32 * ((t) >> 3) * kRowBytes))
 
-      // ---- phase A: S0^T = K0 Q^T -------------------------------------------------------------
-      // (the scheduling fences keep the operand fetches at their distance: left alone, the reads sink next
-      // to their use and every MFMA then waits out a full LDS latency)
+      // The 32 MFMAs of a tile are slots 0..31 (16 for S^T, 16 for O^T); the operand of slot n is fetched from
+      // LDS while slot n - kDist is issued.  The scheduling fences keep that distance: left alone, the reads sink
+      // next to their use and every MFMA then waits out a full LDS latency.
+#define AA_OPERAND_FETCH(n)                          \
+  {                                                  \
+    if ((n) < 16) {                                  \
+      AA_K_FETCH((n) & 15);                          \
+    } else if ((n) < 32) {                           \
+      AA_V_FETCH(((n) - 16) & 15)                    \
+    }                                                \
+  }
+#define AA_S_MFMA(sx, n) sx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[n], qreg[(n) & 7], ((n) & 7) == 0 ? negm : sx, 0, 0, 0)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) AA_K_FETCH(t);
+      for (int n = 0; n < kDist; ++n) AA_OPERAND_FETCH(n)
       AA_FENCE;
+
+      // ---- phase A: S0^T = K0 Q^T (and the next tile's eight loads) -------------------------------
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        AA_K_FETCH(t + 4);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[t], qreg[t], t == 0 ? negm : s0, 0, 0, 0);
-        AA_FETCH_ONE(t)
+      for (int n = 0; n < 8; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_S_MFMA(s0, n);
+        AA_FETCH_ONE(n)
         AA_FENCE;
       }
       AA_STAMP(1)
 
       // ---- phase B: S1^T = K1 Q^T, with the soft-max of S0 between the MFMAs ---------------------
-      AA_K_FETCH(12);
-      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[8], qreg[0], negm, 0, 0, 0);
-      AA_FENCE;
-      AA_K_FETCH(13);
-      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[9], qreg[1], s1, 0, 0, 0);
-      AA_FENCE;
+#pragma unroll
+      for (int n = 8; n < 10; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_S_MFMA(s1, n);
+        AA_FENCE;
+      }
       AA_MASK(s0, 0)
       AA_ROWMAX(s0, mx0)
       const bool moved0 = __any(m_ref + mx0 > m_run);
@@ -393,30 +408,28 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
       AA_FENCE;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if (c < 2) AA_K_FETCH(14 + c);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[10 + c], qreg[2 + c], s1, 0, 0, 0);
-        AA_EXP_CHUNK(s0, pw0, sum0, c)
+      for (int n = 10; n < 14; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_S_MFMA(s1, n);
+        AA_EXP_CHUNK(s0, pw0, sum0, n - 10)
         AA_FENCE;
       }
       l_run += sum0;
-      AA_V_FETCH(0)
-      AA_V_FETCH(1)
-      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[14], qreg[6], s1, 0, 0, 0);
-      AA_FENCE;
-      AA_V_FETCH(2)
-      AA_V_FETCH(3)
-      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[15], qreg[7], s1, 0, 0, 0);
-      AA_FENCE;
+#pragma unroll
+      for (int n = 14; n < 16; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_S_MFMA(s1, n);
+        AA_FENCE;
+      }
       AA_STAMP(2)
 
       // ---- phase C: O^T += V0^T P0^T, with the soft-max of S1 between the MFMAs --------------------
-      AA_V_FETCH(4)
-      AA_PV_MFMA(0, pw0)
-      AA_FENCE;
-      AA_V_FETCH(5)
-      AA_PV_MFMA(1, pw0)
-      AA_FENCE;
+#pragma unroll
+      for (int n = 16; n < 18; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_PV_MFMA(n - 16, pw0)
+        AA_FENCE;
+      }
       if (moved0) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s1[r] -= shift0;
@@ -439,19 +452,19 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
       AA_FENCE;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        AA_V_FETCH(6 + c)
-        AA_PV_MFMA(2 + c, pw0)
-        AA_EXP_CHUNK(s1, pw1, sum1, c)
+      for (int n = 18; n < 22; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_PV_MFMA(n - 16, pw0)
+        AA_EXP_CHUNK(s1, pw1, sum1, n - 18)
         AA_FENCE;
       }
       l_run += sum1;
-      AA_V_FETCH(10)
-      AA_PV_MFMA(6, pw0)
-      AA_FENCE;
-      AA_V_FETCH(11)
-      AA_PV_MFMA(7, pw0)
-      AA_FENCE;
+#pragma unroll
+      for (int n = 22; n < 24; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_PV_MFMA(n - 16, pw0)
+        AA_FENCE;
+      }
       if (moved1) {
 #pragma unroll
         for (int db = 0; db < 4; ++db)
@@ -461,11 +474,13 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 
       // ---- phase D: O^T += V1^T P1^T ---------------------------------------------------------------
 #pragma unroll
-      for (int j = 8; j < 16; ++j) {
-        if (j + 4 < 16) AA_V_FETCH(j + 4)
-        AA_PV_MFMA(j, pw1)
+      for (int n = 24; n < 32; ++n) {
+        AA_OPERAND_FETCH(n + kDist)
+        AA_PV_MFMA(n - 16, pw1)
         AA_FENCE;
       }
+#undef AA_OPERAND_FETCH
+#undef AA_S_MFMA
       AA_STAMP(3)
 #undef AA_K_FETCH
     }

@@ -107,13 +107,17 @@ hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
 // LDS (double-buffered, one barrier per group) together with the groups' thresholds.
 constexpr int kARowStride = 136;  // bf16 per staged pooled-query row: 272 B, conflict-free for row-per-lane 16-byte reads
 
+constexpr int kKB = 2;  // 32-key blocks a wave keeps in registers (2: 64 keys, 64 VGPRs -> two work-groups per CU)
+
 template <int STEP>
-__global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) {
+__global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs p) {
   constexpr int kItems = 32 / STEP;
+  constexpr int kWavesPerTile = 4 / kKB;      // waves that share one 128-key tile
+  constexpr int kTilesPerWg = 4 / kWavesPerTile;
   __shared__ __attribute__((aligned(16))) __bf16 a_lds[2][32 * kARowStride];
   __shared__ __attribute__((aligned(16))) float thr_lds[2][32];
 
-  const int T = blockIdx.x;  // key super-tile (512 keys)
+  const int T = blockIdx.x;  // key super-tile (kTilesPerWg * 128 keys)
   const int kvh = blockIdx.y, b = blockIdx.z;
   const int n_bb = p.n_ctx / p.big_block;
   const int n_t = p.n_ctx / 128;
@@ -123,9 +127,10 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
   const int half = lane >> 5, c32 = lane & 31;
 
   // key tile t is a candidate for big block bb iff 1 <= t <= STEP*bb - 2, i.e. bb >= (t + 2 + STEP - 1) / STEP
-  const int tw = 4 * T + wave;                                   // this wave's key tile
+  const int tw = kTilesPerWg * T + wave / kWavesPerTile;          // this wave's 128-key tile
+  const int kb0 = kKB * (wave % kWavesPerTile);                   // its first 32-key block inside the tile
   const int bb_min_w = tw == 0 ? n_bb : (tw + 2 + STEP - 1) / STEP;  // tile 0 is never a candidate
-  const int t_first = T == 0 ? 1 : 4 * T;                         // first candidate tile of the work-group
+  const int t_first = T == 0 ? 1 : kTilesPerWg * T;               // first candidate tile of the work-group
   const int bb_lo = (t_first + 2 + STEP - 1) / STEP;              // smallest big block any wave needs
   if (bb_lo >= n_bb) return;
   const int group = p.n_q_heads / p.n_kv_heads;
@@ -133,10 +138,10 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
   const int n_groups = (n_items + kItems - 1) / kItems;
 
   const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
-  bf16x8 kreg[4][8];
+  bf16x8 kreg[kKB][8];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb) {
-    const __bf16* row = kp + (int64_t)(tw * 128 + 32 * kb + c32) * p.k_sn + 8 * half;
+  for (int kb = 0; kb < kKB; ++kb) {
+    const __bf16* row = kp + (int64_t)(tw * 128 + 32 * (kb0 + kb) + c32) * p.k_sn + 8 * half;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
   }
@@ -144,6 +149,7 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
   // staging: thread t carries 32 bytes (chunks 2*(t&7), 2*(t&7)+1) of pooled row t>>3 of the group; row r of a
   // group is pooled row (r % STEP) of item grp*kItems + r/STEP; threads 0..31 also carry the row's threshold
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   u32x4 st0, st1;
   float st_thr = 0.f;
   auto stage_load = [&](const int grp) {
@@ -195,9 +201,9 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
         thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
         thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
       }
-      uint32_t words[kItems][4];
+      uint32_t words[kItems][kKB];
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
+      for (int kb = 0; kb < kKB; ++kb) {
         const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         floatx16 c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kreg[kb][0], zero, 0, 0, 0);
 #pragma unroll
@@ -220,8 +226,12 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
             const int item = grp * kItems + it;
             const int hq = kvh * group + item % group;
             const int bb = bb_lo + item / group;
-            uint4 w = {words[it][0], words[it][1], words[it][2], words[it][3]};
-            *reinterpret_cast<uint4*>(p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + tw) * 4) = w;
+            uint32_t* dst = p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + tw) * 4 + kb0;
+            if (kKB == 4) {
+              *reinterpret_cast<u32x4*>(dst) = u32x4{words[it][0], words[it][1], words[it][kKB - 2], words[it][kKB - 1]};
+            } else {
+              *reinterpret_cast<u32x2*>(dst) = u32x2{words[it][0], words[it][1]};
+            }
           }
         }
       }
@@ -233,7 +243,7 @@ __global__ void __launch_bounds__(256) select_scores_kernel(const SelectArgs p) 
 
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
   const int step = a.big_block / a.block_size;
-  const dim3 grid(a.n_ctx / 512, a.n_kv_heads, a.batch);
+  const dim3 grid(a.n_ctx / (128 * kKB), a.n_kv_heads, a.batch);
   if (step == 16) hipLaunchKernelGGL(select_scores_kernel<16>, grid, dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(select_scores_kernel<32>, grid, dim3(256), 0, stream, a);
   return hipGetLastError();

@@ -143,3 +143,29 @@ def test_synthetic_generator_properties():
     pw = stripe_positions(131072, 655, "powerlaw", g)
     assert pw.numel() == 655 and pw.unique().numel() == 655 and pw.min() >= 1 and pw.max() < 131072
     assert (pw < 131072 // 4).sum() > 655 * 0.4  # density decays with position (uniform would give 25%)
+
+
+def test_analysis_tools_on_cpu():
+    """get_deff metrics and the token-level ideal (plain torch, no kernel involved)."""
+    import torch
+    from anchor_attn.src.ops.sparse_attn_with_pytorch import sparse_attn_with_torch
+    from my_utils.ops_util import get_deff
+    x = torch.tensor([1.0, -2.0, 0.0, 4.0])
+    y = torch.tensor([1.0005, -2.5, 0.00005, 10.0])
+    mean_err, strict, loose, m = get_deff(x, y, verbose=False)
+    assert abs(float(mean_err) - (0.0005 + 0.5 + 0.00005 + 6.0) / 4) < 1e-6
+    assert strict == 0.5 and loose == 0.75  # -2.5 is within 30% of -2; 10 is not within 30% of 4
+    assert m["abs_error_ratios"]["<= 0.1"] == 0.5 and 0 < m["cosine_similarity"] < 1
+    with pytest.raises(ValueError):
+        get_deff(x, y[:2])
+    # theta large: the ideal keeps every causal key and equals dense attention; GQA heads are expanded
+    torch.manual_seed(0)
+    q, k, v = torch.randn(1, 4, 70, 16), torch.randn(1, 2, 70, 16), torch.randn(1, 2, 70, 16)
+    out, ratio = sparse_attn_with_torch(q, k, v, diff_anchor=1e4, return_computational_ratio=True, chunk_size=32)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k.repeat_interleave(2, 1), v.repeat_interleave(2, 1), is_causal=True)
+    assert ratio == 1.0 and torch.allclose(out, ref, atol=1e-5)
+    # theta = 0 keeps only each row's maximum: output is the value row of the arg-max key
+    out0, r0 = sparse_attn_with_torch(q, k, v, diff_anchor=0.0, return_computational_ratio=True)
+    s = (q @ k.repeat_interleave(2, 1).transpose(-1, -2)).masked_fill(torch.triu(torch.ones(70, 70, dtype=torch.bool), 1), float("-inf"))
+    want = torch.gather(v.repeat_interleave(2, 1), 2, s.argmax(-1, keepdim=True).expand(-1, -1, -1, 16))
+    assert torch.allclose(out0, want, atol=1e-5) and abs(r0 - 70 / (70 * 71 / 2)) < 1e-9
