@@ -35,7 +35,8 @@ def _workspace(B, H, N, D, block_size, step, device):
 
 
 def _anchor_attn(Q, K, V, sm_scale=None, block_size=64, step=16, difference=100, return_sparsity_ratio=False,
-                 BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, out=None, scale_mode=_hip.AA_SCALE_BF16_CHAIN):
+                 BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, out=None, scale_mode=_hip.AA_SCALE_BF16_CHAIN,
+                 geometry=_hip.AA_GEOMETRY_AS_RUN):
     """All three stages on the current stream, one C call (``difference`` is in the log2 domain
     here, as in the reference's private function, anchor_attn_v4.py:226-273)."""
     B, H, N, D = Q.shape
@@ -49,7 +50,7 @@ def _anchor_attn(Q, K, V, sm_scale=None, block_size=64, step=16, difference=100,
     _hip.check(_hip.lib().aa_anchor_attn_fwd(
         *_hip.t3(Q), *_hip.t3(K), *_hip.t3(V), *_hip.t3(output),
         ws.data_ptr(), ws.numel(), counts.data_ptr() if counts is not None else None,
-        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), float(difference / LOG2E), scale_mode, _stream()))
+        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), float(difference / LOG2E), scale_mode, int(geometry), _stream()))
     if return_sparsity_ratio:
         return output, _ratio(counts, B, H, N, block_size, step)
     return output, 1.0
@@ -101,9 +102,13 @@ def anchor_attn_without_anchor(Q, K, V, sm_scale: float = None, block_size: int 
 
 
 def anchor_attn(Q, K, V, sm_scale: float = None, block_size: int = 128, step: int = 16, difference: float = 12,
-                return_computational_ratio: bool = True, out: torch.Tensor = None):
+                return_computational_ratio: bool = True, out: torch.Tensor = None, strict_reference: bool = True):
     """Sparse prefill attention.  ``Q`` ``[B,H,N,D]`` bf16; ``K``/``V`` ``[B,H or H_kv,N,D]``;
-    returns ``out`` or ``(out, ratio)`` exactly like the reference."""
+    returns ``out`` or ``(out, ratio)`` exactly like the reference.
+
+    ``strict_reference=False`` (analysis only, never the default) lets stage 2 choose from ``[S, bb*S)``
+    - the range of the reference's fused variant, anchor_fuse_step_1_2_v2.py:152 - instead of the as-run
+    ``[block_size, bb*S - block_size)``: no key is attended twice and none is left out."""
     difference *= LOG2E
     Q, K, V = _prepare(Q, K, V)
     assert Q.stride(-1) == 1 and K.stride(-1) == 1 and V.stride(-1) == 1, \
@@ -118,7 +123,8 @@ def anchor_attn(Q, K, V, sm_scale: float = None, block_size: int = 128, step: in
     B, H, N, D = Q.shape
     sm_scale = sm_scale if sm_scale else 1.0 / (D ** 0.5)
     sparse_output, sparse_ratio = _anchor_attn(Q, K, V, sm_scale, block_size, step, difference,
-                                               return_computational_ratio, out=out)
+                                               return_computational_ratio, out=out,
+                                               geometry=_hip.AA_GEOMETRY_AS_RUN if strict_reference else _hip.AA_GEOMETRY_INTENDED)
     if return_computational_ratio:
         from my_utils import Logger
         Logger.log(f"anchor sparse_ratio:{sparse_ratio}")

@@ -71,7 +71,7 @@ def pool_q_anchor(Q, M_buffer, block_size):
     return qbar, abar
 
 
-def select_stripes_packed(Q, K, M_buffer, block_size, step, theta, B, H, N, D, sm_scale):
+def select_stripes_packed(Q, K, M_buffer, block_size, step, theta, B, H, N, D, sm_scale, geometry=_hip.AA_GEOMETRY_AS_RUN):
     """Stage 2 with packed outputs: ``(coords int32 [B,H,entries_per_head], counts int32
     [B,H,N/S,1])``; ``theta`` is already in the log2 domain, as the reference passes it."""
     _check_inputs(Q, K)
@@ -85,7 +85,7 @@ def select_stripes_packed(Q, K, M_buffer, block_size, step, theta, B, H, N, D, s
     counts = torch.empty((B, H, n_bb, 1), dtype=torch.int32, device=Q.device)
     _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(K), mask.data_ptr(), coords.data_ptr(),
                                     counts.data_ptr(), B, H, K.shape[1], N, D, block_size, step,
-                                    float(sm_scale), float(theta), _stream()))
+                                    float(sm_scale), float(theta), int(geometry), _stream()))
     return coords, counts
 
 

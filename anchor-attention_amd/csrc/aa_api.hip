@@ -209,9 +209,13 @@ int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, float sm_scale, float theta_log2, void* stream) {
+                     int block_size, int step, float sm_scale, float theta_log2, int geometry, void* stream) {
   const char* who = "aa_stage2_select";
   int rc;
+  if (geometry != AA_GEOMETRY_AS_RUN && geometry != AA_GEOMETRY_INTENDED) {
+    set_error("%s: geometry %d is neither AA_GEOMETRY_AS_RUN nor AA_GEOMETRY_INTENDED", who, geometry);
+    return AA_EBADARG;
+  }
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
   if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
   if ((rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar")) || (rc = check_ptr(mask_ws, who, "mask_ws")) ||
@@ -227,6 +231,8 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.big_block = block_size * step; a.block_size = block_size;
   a.scale2 = (float)((double)sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
+  a.tile_lo = geometry == AA_GEOMETRY_AS_RUN ? 1 : step;
+  a.tile_slack = geometry == AA_GEOMETRY_AS_RUN ? 2 : 1;
   if ((rc = check_launch(launch_select_thresholds(a, (hipStream_t)stream), who))) return rc;
   if ((rc = check_launch(launch_select_scores(a, (hipStream_t)stream), who))) return rc;
   return check_launch(launch_select_compact(a, (hipStream_t)stream), who);
@@ -273,7 +279,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                       int block_size, int step, float sm_scale, float theta, int scale_mode,
+                       int block_size, int step, float sm_scale, float theta, int scale_mode, int geometry,
                        void* stream) {
   const char* who = "aa_anchor_attn_fwd";
   int rc;
@@ -300,7 +306,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   // theta -> log2 domain: a double product rounded to float32 (the definition multiplies a Python float)
   const float theta_log2 = (float)((double)theta * 1.44269504);
   if ((rc = aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, mask, coords, counts, batch, n_q_heads, n_kv_heads, n_ctx,
-                             head_dim, block_size, step, sm_scale, theta_log2, stream)))
+                             head_dim, block_size, step, sm_scale, theta_log2, geometry, stream)))
     return rc;
   if ((rc = aa_stage3_sparse_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, coords, counts, M, L, acc, out,
                                  o_sb, o_sh, o_sn, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale,

@@ -126,12 +126,14 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, c32 = lane & 31;
 
-  // key tile t is a candidate for big block bb iff 1 <= t <= STEP*bb - 2, i.e. bb >= (t + 2 + STEP - 1) / STEP
+  // key tile t is a candidate for big block bb iff tile_lo <= t <= STEP*bb - tile_slack,
+  // i.e. t >= tile_lo and bb >= (t + tile_slack + STEP - 1) / STEP
   const int tw = kTilesPerWg * T + wave / kWavesPerTile;          // this wave's 128-key tile
   const int kb0 = kKB * (wave % kWavesPerTile);                   // its first 32-key block inside the tile
-  const int bb_min_w = tw == 0 ? n_bb : (tw + 2 + STEP - 1) / STEP;  // tile 0 is never a candidate
-  const int t_first = T == 0 ? 1 : kTilesPerWg * T;               // first candidate tile of the work-group
-  const int bb_lo = (t_first + 2 + STEP - 1) / STEP;              // smallest big block any wave needs
+  const int bb_min_w = tw < p.tile_lo ? n_bb : (tw + p.tile_slack + STEP - 1) / STEP;
+  if (kTilesPerWg * T + kTilesPerWg - 1 < p.tile_lo) return;      // no tile of the work-group is ever a candidate
+  const int t_first = max(p.tile_lo, kTilesPerWg * T);            // first candidate tile of the work-group
+  const int bb_lo = (t_first + p.tile_slack + STEP - 1) / STEP;   // smallest big block any wave needs
   if (bb_lo >= n_bb) return;
   const int group = p.n_q_heads / p.n_kv_heads;
   const int n_items = group * (n_bb - bb_lo);
@@ -257,7 +259,7 @@ __global__ void __launch_bounds__(64) select_compact_kernel(const SelectArgs p) 
   const int n_t = p.n_ctx / 128;
   const int step = p.big_block / p.block_size;
   const int64_t bh = (int64_t)b * p.n_q_heads + h;
-  const int t_lo = 1, t_hi = step * bb - 2;  // candidate key tiles, inclusive
+  const int t_lo = p.tile_lo, t_hi = step * bb - p.tile_slack;  // candidate key tiles, inclusive
   int base = 0;
   if (t_hi >= t_lo) {
     const int n_words = 4 * (t_hi - t_lo + 1);

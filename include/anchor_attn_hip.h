@@ -40,6 +40,14 @@ extern "C" {
 #define AA_SCALE_BF16_CHAIN 0
 #define AA_SCALE_FP32 1
 
+/* Which keys stage 2 may select for big block bb.  AA_GEOMETRY_AS_RUN is what the reference's operator does
+ * (get_mask_test.py:93-94): [block_size, bb*S - block_size) - keys below S are then attended twice (stage 1
+ * already covers [0,S)) and the last block_size keys before the big block never.  AA_GEOMETRY_INTENDED is the
+ * range the reference's fused variant walks (anchor_fuse_step_1_2_v2.py:152, init_limit .. local_start):
+ * [S, bb*S), no overlap and no gap.  Never the default; it exists to measure what the as-run quirks cost. */
+#define AA_GEOMETRY_AS_RUN 0
+#define AA_GEOMETRY_INTENDED 1
+
 int aa_version(void);
 const char* aa_last_error(void);
 
@@ -88,14 +96,15 @@ int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, co
 /* Replaces anchor_attn_step_2 / get_q_mask / get_q_mask_triton (anchor_step_1_2_v2.py:199-210,
  * get_mask_test.py:7-159): key j in [block_size, bb*S - block_size) is selected for big block bb
  * iff for one of its pooled rows i  float(bf16(dot(qbar_i,k_j) * sm_scale*1.44269504)) + theta_log2
- * >= float(abar_i).  theta_log2 is theta * 1.44269504 (anchor_attn_v4.py:298).
+ * >= float(abar_i).  theta_log2 is theta * 1.44269504 (anchor_attn_v4.py:298).  geometry: AA_GEOMETRY_* (the
+ * candidate range above is the as-run one).
  * mask_ws: scratch of aa_mask_words() uint32.  Outputs: coords (packed, see above) and
  * counts [B,Hq,N/S] int32.  Deterministic: no atomics, lists are ascending. */
 int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, float sm_scale, float theta_log2, void* stream);
+                     int block_size, int step, float sm_scale, float theta_log2, int geometry, void* stream);
 
 /* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
  * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
@@ -122,7 +131,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                       int block_size, int step, float sm_scale, float theta, int scale_mode,
+                       int block_size, int step, float sm_scale, float theta, int scale_mode, int geometry,
                        void* stream);
 
 /* ---- dense causal baseline on the same MFMA core --------------------------------------------

@@ -213,8 +213,12 @@ def stage2_select(
     theta: float,
     block_size: int = 128,
     step: int = 16,
+    strict_reference: bool = True,
 ) -> Tuple[List[List[List[np.ndarray]]], np.ndarray]:
     """Difference-aware stripe identification (``get_q_mask_triton``).
+
+    ``strict_reference=False`` replaces the as-run candidate range by ``[S, bb*S)``, the range the
+    reference's fused variant walks (anchor_fuse_step_1_2_v2.py:152); everything else is unchanged.
 
     For big block ``bb`` the candidate keys are ``[block_size, bb*S - block_size)``
     (get_mask_test.py:93-94); key ``j`` is selected iff for some pooled row ``i`` of the big
@@ -240,7 +244,7 @@ def stage2_select(
             abar, _ = pooled_anchors(M[b, h], block_size)
             per_h = []
             for bb in range(n_bb):
-                lo, hi = block_size, bb * S - block_size
+                lo, hi = (block_size, bb * S - block_size) if strict_reference else (S, bb * S)
                 if hi <= lo:
                     per_h.append(np.zeros(0, np.int32))
                     continue
@@ -347,6 +351,7 @@ def anchor_attn_reference(
     step: int = 16,
     difference: float = 12.0,
     stage1_scale_mode: str = "bf16_chain",
+    strict_reference: bool = True,
 ) -> OracleResult:
     """The operator end to end, as ``anchor_attn`` runs it (anchor_attn_v4.py:291-324)."""
     B, Hq, N, D = Q.shape
@@ -355,7 +360,7 @@ def anchor_attn_reference(
     if not sm_scale:
         sm_scale = 1.0 / math.sqrt(D)
     M, L, Acc = stage1_anchor(Q, K, V, sm_scale, block_size, step, stage1_scale_mode)
-    coords, counts = stage2_select(Q, K, M, sm_scale, difference, block_size, step)
+    coords, counts = stage2_select(Q, K, M, sm_scale, difference, block_size, step, strict_reference)
     out = stage3_sparse(Q, K, V, coords, counts, M, L, Acc, sm_scale, block_size, step)
     ratio = sparsity_ratio(counts, B, Hq, N, block_size, step)
     return OracleResult(out, M, L, Acc, coords, counts, ratio)

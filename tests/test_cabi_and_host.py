@@ -61,9 +61,9 @@ def test_error_codes_without_touching_the_gpu():
     assert dense(p, 2, 2, 2000, 128) == 2
     assert dense(p + 2, 2, 2, 2048, 128) == 3 and b"aligned" in lib.aa_last_error()
     assert dense(p, 2, 2, 2048, 128, qs=(s[0], s[1], 132)) == 3
-    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1024, None, 1, 2, 2, 2048, 128, 128, 16, 0.1, 12.0, 0, None)
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1024, None, 1, 2, 2, 2048, 128, 128, 16, 0.1, 12.0, 0, 0, None)
     assert rc == 1 and b"workspace" in lib.aa_last_error()
-    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, None)
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, 0, None)
     assert rc == 2 and b"multiple" in lib.aa_last_error()
     rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 8, 0.1, 0, None)
     assert rc == 2 and b"step" in lib.aa_last_error()

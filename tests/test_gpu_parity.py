@@ -333,6 +333,40 @@ def test_constant_values_at_32k(mods):
     assert err.max() <= 2e-2
 
 
+def test_intended_geometry_mode(mods):
+    """strict_reference=False against the oracle in the same mode; with theta -> +inf it is plain causal attention
+    (no key twice, none left out), and no selected index lies below the big block."""
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(4 * S, 4, 2, 96, seed=71)
+    Q, K, V = _np(q, k, v)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    res = ao.anchor_attn_reference(Q, K, V, difference=12.0, strict_reference=False)
+    out, ratio = v4.anchor_attn(qd, kd, vd, difference=12.0, strict_reference=False)
+    err = np.abs(out.float().cpu().numpy() - res.out)
+    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM, geometry=hip.AA_GEOMETRY_INTENDED)
+    got, got_counts = _packed_lists(hip, coords, counts, N)
+    excused = 0
+    for h in range(H):
+        for bb in range(N // S):
+            g, w = got[0][h][bb], res.coords[0][h][bb]
+            assert g.size == 0 or (g[0] >= S and g[-1] < bb * S)
+            excused += np.setxor1d(g, w).size
+    assert excused <= 4 and got_counts[:, :, :2].sum() == 0 and got_counts.sum() > 0
+    assert abs(float(ratio) - got_counts.sum() / ((B * H * N * N / (BS * STEP)) // 2)) < 1e-6
+    full, _ = v4.anchor_attn(qd, kd, vd, difference=1e4, strict_reference=False)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    e = (full.cpu().double() - ref).abs()
+    # (looser than the oracle bound: the stage-1 bf16 scale chain is part of the operator, not of plain attention)
+    assert e.max() < 4e-2 and e.mean() < 2e-3
+    lib = hip.lib()
+    assert lib.aa_stage2_select(1, 1, 1, 0, 0, 128, 1, 1, 1, 1, 2, 2, 2048, 128, 128, 16, 0.1, 1.0, 5, None) == 1
+    assert b"geometry" in lib.aa_last_error()
+
+
 def test_full_size_128k_sampled_parity(mods):
     """BASELINE config 2 (Llama-3.1-8B layer, 128k tokens, 32/8 heads) through all three stages; sampled
     rows and sampled (head, big block) pairs are recomputed on the host in float64 / with the oracle's

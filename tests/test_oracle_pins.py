@@ -289,3 +289,23 @@ def test_reference_layout_packing(small):
     assert tc.shape == (1, 2, 3, Q.shape[2]) and tc.dtype == np.int32
     c = res.coords[0][1][2]
     assert np.array_equal(tc[0, 1, 2, : c.size], c) and not tc[0, 1, 2, c.size :].any()
+
+
+def test_intended_geometry_candidate_range_and_dense_limit():
+    """strict_reference=False: candidates are exactly [S, bb*S) (theta -> +inf selects all of them), and then the
+    operator has no double-counted key and no gap, so it equals plain causal attention - which the as-run
+    geometry does not (keys below S counted twice, the last 128 keys before each big block missing)."""
+    rng = np.random.default_rng(11)
+    N, H = 3 * 2048, 1
+    Q = ao.rn16(rng.standard_normal((1, H, N, 128)).astype(np.float32))
+    K = ao.rn16(rng.standard_normal((1, H, N, 128)).astype(np.float32))
+    V = ao.rn16(rng.standard_normal((1, H, N, 128)).astype(np.float32))
+    res = ao.anchor_attn_reference(Q, K, V, difference=1e4, strict_reference=False)
+    for bb in range(3):
+        want = np.arange(2048, bb * 2048, dtype=np.int32) if bb >= 2 else np.zeros(0, np.int32)
+        assert np.array_equal(res.coords[0][0][bb], want)
+    q = torch.from_numpy(Q).double(); k = torch.from_numpy(K).double(); v = torch.from_numpy(V).double()
+    dense = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True).numpy()
+    assert np.abs(res.out - dense).max() < 2e-2 and np.abs(res.out - dense).mean() < 2e-3
+    as_run = ao.anchor_attn_reference(Q, K, V, difference=1e4)
+    assert np.abs(as_run.out[0, 0, 2 * 2048:] - dense[0, 0, 2 * 2048:]).max() > 5e-2
