@@ -108,17 +108,20 @@ __device__ __forceinline__ void load16_to_lds(const char* base, const uint32_t b
 template <int MODE>
 __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, const char* vb, const uint32_t k_row_bytes,
                                                const uint32_t v_row_bytes, const uint32_t k_col, const uint32_t v_col, const int key0,
-                                               const int tid, const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v) {
+                                               const int tid, const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v,
+                                               const uint32_t (&k_voff)[4], const uint32_t (&v_voff)[4]) {
   const int j = n >> 1;  // load n: K (even n) or V (odd n) rows 16*j + ...
-  const int row = (tid >> 4) + 16 * j;
-  uint32_t key;
   if (MODE == kSparse) {
-    key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
+    const int row = (tid >> 4) + 16 * j;
+    const uint32_t key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
+    if ((n & 1) == 0) load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
+    else load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
   } else {
-    key = (uint32_t)(key0 + row);
+    // consecutive keys: the tile's first row goes into the (scalar) base address, the thread's row and chunk
+    // inside the tile are loop-invariant vector offsets - no vector arithmetic per tile
+    if ((n & 1) == 0) load16_to_lds(kb + (uint64_t)(uint32_t)key0 * k_row_bytes, k_voff[j], lds_k + 16 * j * kRowBytes);
+    else load16_to_lds(vb + (uint64_t)(uint32_t)key0 * v_row_bytes, v_voff[j], lds_v + 16 * j * kRowBytes);
   }
-  if ((n & 1) == 0) load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
-  else load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
 }
 
 template <int MODE>
@@ -195,10 +198,17 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const uint32_t k_col = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15)) * 16u;
   const uint32_t v_col = (uint32_t)((tid & 15) ^ (((tid >> 4) & 7) << 1)) * 16u;
   const uint32_t lds_k0 = lds_addr(sm.t.k[0]) + wave * 4 * kRowBytes, lds_v0 = lds_addr(sm.t.v[0]) + wave * 4 * kRowBytes;
+  uint32_t k_voff[4], v_voff[4];  // byte offset of this thread's chunk of tile row (tid >> 4) + 16*j from the tile's first row
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    k_voff[j] = ((tid >> 4) + 16 * j) * k_row_bytes + k_col;
+    v_voff[j] = ((tid >> 4) + 16 * j) * v_row_bytes + v_col;
+  }
   if (n_tiles > 0) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0);
+      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0,
+                           k_voff, v_voff);
   }
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
@@ -338,7 +348,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #else
 #define AA_FETCH_ONE(n)                                                                                               \
   tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,   \
-                                  lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes);
+                                  lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes, k_voff, v_voff);
 #endif
 
     AA_STAMP(0)
