@@ -62,7 +62,7 @@ int check_dims(const Dims& d, const char* who) {
   return AA_OK;
 }
 
-int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, const char* who, const char* name) {
+int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, int n_ctx, const char* who, const char* name) {
   if (ptr == nullptr) {
     set_error("%s: %s is NULL", who, name);
     return AA_EBADARG;
@@ -77,6 +77,11 @@ int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, const char
   }
   if (sn > (int64_t)1 << 14) {  // the kernels address rows of one head with 32-bit byte offsets
     set_error("%s: %s row stride %lld is larger than 16384 elements", who, name, (long long)sn);
+    return AA_EUNSUPPORTED;
+  }
+  if ((int64_t)n_ctx * sn * 2 > (int64_t)0xffffffffLL) {
+    set_error("%s: %s spans %lld bytes per head (n_ctx %d x row stride %lld elements); the kernels address one head with 32-bit byte offsets",
+              who, name, (long long)n_ctx * sn * 2, n_ctx, (long long)sn);
     return AA_EUNSUPPORTED;
   }
   return AA_OK;
@@ -171,9 +176,9 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   const char* who = "aa_stage1_anchor_fwd";
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
   if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag"))) return rc;
   if (scale_mode != AA_SCALE_BF16_CHAIN && scale_mode != AA_SCALE_FP32) {
     set_error("%s: unknown scale_mode %d", who, scale_mode);
@@ -196,7 +201,7 @@ int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, co
   const char* who = "aa_pool_q_anchor";
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_q_heads, n_ctx, head_dim, block_size, 16}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar"))) return rc;
   PoolArgs a = {};
   a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
@@ -217,7 +222,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
     return AA_EBADARG;
   }
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
   if ((rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar")) || (rc = check_ptr(mask_ws, who, "mask_ws")) ||
       (rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")))
     return rc;
@@ -249,10 +254,10 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   const char* who = "aa_stage3_sparse_fwd";
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
-  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, who, "out"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, who, "out"))) return rc;
   if ((rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")) || (rc = check_ptr(M, who, "M")) ||
       (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag")))
     return rc;
@@ -335,10 +340,10 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   Dims d = {batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16};
   d.n_ctx = 2048;  // only the generic checks; divisibility by the big block does not apply here
   if ((rc = check_dims(d, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, who, "v"))) return rc;
-  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, who, "out"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, who, "out"))) return rc;
   FlashArgs a = {};
   a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
   a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;

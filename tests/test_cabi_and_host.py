@@ -65,6 +65,9 @@ def test_error_codes_without_touching_the_gpu():
     assert rc == 1 and b"workspace" in lib.aa_last_error()
     rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, 0, None)
     assert rc == 2 and b"multiple" in lib.aa_last_error()
+    big = (s[0], s[1], 16384)  # 2^20 rows x 32 KiB per row does not fit 32-bit byte offsets
+    rc = lib.aa_stage1_anchor_fwd(p, *big, p, *s, p, *s, p, p, p, 1, 2, 2, 1 << 20, 128, 128, 16, 0.1, 0, None)
+    assert rc == 2 and b"32-bit" in lib.aa_last_error()
     rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 8, 0.1, 0, None)
     assert rc == 2 and b"step" in lib.aa_last_error()
     rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 7, None)

@@ -367,6 +367,45 @@ def test_intended_geometry_mode(mods):
     assert b"geometry" in lib.aa_last_error()
 
 
+def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples):
+    """Stages 1 and 3 on sampled (head, row) pairs, recomputed in float64 on the host (P rounded to bf16 as the
+    kernels do) from the kernel's own index lists; returns the per-row max errors."""
+    N = q.shape[2]
+    group = q.shape[1] // k.shape[1]
+    errs = []
+    for h, r in samples:
+        bb = r // S
+        kv = h // group
+        keys1 = np.unique(np.concatenate([np.arange(0, min(S, r + 1)), np.arange(bb * S, r + 1)]))
+        K1 = k[0, kv, keys1].double().cpu().numpy()
+        V1 = v[0, kv, keys1].double().cpu().numpy()
+        qrow = q[0, h, r].float().cpu().numpy()
+        q1 = ao.q1_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        s1 = K1 @ q1
+        m1 = s1.max()
+        p1 = np.exp2(s1 - m1)
+        l1 = p1.sum()
+        a1 = ao.rn16(p1.astype(np.float32)).astype(np.float64) @ V1
+        assert abs(float(M[0, h, r]) - m1) < 3e-4
+        assert abs(float(L[0, h, r]) - l1) / l1 < 1e-3
+        lst = index_list(h, bb)
+        q3 = ao.q3_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        if lst.size:
+            K3 = k[0, kv, lst].double().cpu().numpy()
+            V3 = v[0, kv, lst].double().cpu().numpy()
+            s3 = K3 @ q3
+            m = max(m1, s3.max())
+            p3 = np.exp2(s3 - m)
+            num = a1 * np.exp2(m1 - m) + ao.rn16(p3.astype(np.float32)).astype(np.float64) @ V3
+            den = l1 * np.exp2(m1 - m) + p3.sum()
+        else:
+            num, den = a1, l1
+        err = np.abs(out[0, h, r].double().cpu().numpy() - num / den)
+        assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (h, r, err.max(), err.mean())
+        errs.append(err.max())
+    return errs
+
+
 def test_full_size_128k_sampled_parity(mods):
     """BASELINE config 2 (Llama-3.1-8B layer, 128k tokens, 32/8 heads) through all three stages; sampled
     rows and sampled (head, big block) pairs are recomputed on the host in float64 / with the oracle's
@@ -407,38 +446,42 @@ def test_full_size_128k_sampled_parity(mods):
             d_ = ao.stage2_flip_distance(qbar, abar, mean, k[0, h // group, int(j)].float().cpu().numpy(), SM, theta)
             assert d_ < BAND, (h, bb, int(j), d_)
         assert np.setxor1d(got, want).size <= 3
-    # ---- stages 1 and 3 on sampled rows (float64 on the host; P rounded to bf16 as the kernels do)
-    out_rows = []
-    for h, r in [(0, 0), (0, N - 1), (5, 2047), (9, 2048), (17, 70000), (31, N - 2048), (26, int(rng.integers(S, N)))]:
-        bb = r // S
-        kv = h // group
-        keys1 = np.unique(np.concatenate([np.arange(0, min(S, r + 1)), np.arange(bb * S, r + 1)]))
-        K1 = k[0, kv, keys1].double().cpu().numpy()
-        V1 = v[0, kv, keys1].double().cpu().numpy()
-        qrow = q[0, h, r].float().cpu().numpy()
-        q1 = ao.q1_scale_chain(qrow[None], SM)[0].astype(np.float64)
-        s1 = K1 @ q1
-        m1 = s1.max()
-        p1 = np.exp2(s1 - m1)
-        l1 = p1.sum()
-        a1 = ao.rn16(p1.astype(np.float32)).astype(np.float64) @ V1
-        assert abs(float(M[0, h, r]) - m1) < 3e-4
-        assert abs(float(L[0, h, r]) - l1) / l1 < 1e-3
-        lst = index_list(h, bb)
-        q3 = ao.q3_scale_chain(qrow[None], SM)[0].astype(np.float64)
-        if lst.size:
-            K3 = k[0, kv, lst].double().cpu().numpy()
-            V3 = v[0, kv, lst].double().cpu().numpy()
-            s3 = K3 @ q3
-            m = max(m1, s3.max())
-            p3 = np.exp2(s3 - m)
-            num = a1 * np.exp2(m1 - m) + ao.rn16(p3.astype(np.float32)).astype(np.float64) @ V3
-            den = l1 * np.exp2(m1 - m) + p3.sum()
-        else:
-            num, den = a1, l1
-        want_row = num / den
-        got_row = out[0, h, r].double().cpu().numpy()
-        err = np.abs(got_row - want_row)
-        assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (h, r, err.max(), err.mean())
-        out_rows.append(err.max())
+    # ---- stages 1 and 3 on sampled rows
+    samples = [(0, 0), (0, N - 1), (5, 2047), (9, 2048), (17, 70000), (31, N - 2048), (26, int(rng.integers(S, N)))]
+    out_rows = _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples)
     assert len(out_rows) == 7
+
+
+def test_maximum_context_one_million_tokens(mods):
+    """The largest context the library accepts (2^20 tokens, 512 big blocks), one head: sampled rows against the
+    float64 host recomputation, index lists ascending and inside their candidate range, constant V => constant
+    output, and one more token than the limit is refused."""
+    hip, v4, st, ao = mods
+    from anchor_attn.synthetic import make_qkv
+    N = 1 << 20
+    q, k, v, _ = make_qkv(N, 1, 1, n_stripes=2048, seed=5, stripe_dist="powerlaw")
+    q, k, v = q.cuda(), k.cuda(), v.cuda()
+    L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, 1, 1, N, D, SM)
+    coords, counts = st.select_stripes_packed(q, k, M, BS, STEP, 12.0 * LOG2E, 1, 1, N, D, SM)
+    out = v4._stage3(q, k, v, coords, counts, L, M, Acc, SM, BS, STEP)
+    fused, ratio = v4.anchor_attn(q, k, v)
+    assert torch.equal(out, fused) and 0 < float(ratio) < 0.05
+    lib = hip.lib()
+    cnt = counts.reshape(N // S).cpu().numpy()
+    flat = coords.reshape(-1)
+
+    def index_list(h, bb):
+        off = lib.aa_coords_offset(bb, BS, STEP)
+        return flat[off:off + int(cnt[bb])].cpu().numpy()
+
+    for bb in (1, 2, 255, 511):
+        lst = index_list(0, bb)
+        assert np.all(np.diff(lst) > 0) and (lst.size == 0 or (lst[0] >= BS and lst[-1] < bb * S - BS))
+    assert cnt[0] == 0 and cnt[511] > 0
+    _check_sampled_rows(ao, q, k, v, M, L, out, index_list, [(0, N - 1), (0, N - 2048), (0, 600000), (0, 2048 * 300 + 5)])
+    row = torch.linspace(-1, 1, D).to(torch.bfloat16).cuda()
+    oc = v4.anchor_attn(q, k, row.expand_as(v).contiguous(), return_computational_ratio=False)
+    assert (oc.float() - row.float()).abs().max() < 2e-2
+    with pytest.raises(hip.AnchorAttnHipError):
+        too_long = torch.empty(1, 1, N + S, D, dtype=torch.bfloat16, device="cuda")
+        v4.anchor_attn(too_long, too_long, too_long)
