@@ -303,6 +303,39 @@ def test_repeatable_bit_for_bit(mods, llama_small):
     assert torch.equal(c, a[0])
 
 
+def test_side_stream_and_graph_replay(mods, llama_small):
+    """Every launch goes to the caller's stream and the library neither allocates nor synchronises, so the whole
+    operator can run on a side stream and be captured in a HIP graph; each replay (with eager work and new
+    inputs between replays) must equal the eager result bit for bit."""
+    hip, v4, st, ao = mods
+    (q, k, v), _, _ = llama_small
+    base = v4.anchor_attn(q, k, v, return_computational_ratio=False)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        o_side = v4.anchor_attn(q, k, v, return_computational_ratio=False)
+    side.synchronize()
+    assert torch.equal(o_side, base)
+    sq, sk, sv = q.clone(), k.clone(), v.clone()
+    s_out = torch.empty_like(q)
+    with torch.cuda.stream(side):  # warm-up outside the capture
+        v4.anchor_attn(sq, sk, sv, return_computational_ratio=False, out=s_out)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        v4.anchor_attn(sq, sk, sv, return_computational_ratio=False, out=s_out)
+    for rep in range(3):
+        if rep:
+            sv.copy_(torch.roll(v, rep, dims=2))      # new values, same selection
+            sq.copy_(q * (1.0 + 0.01 * rep))          # new queries: anchors and selection move too
+        want = v4.anchor_attn(sq, sk, sv, return_computational_ratio=False)
+        torch.cuda.synchronize()
+        s_out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(s_out, want), f"replay {rep} differs from the eager result"
+
+
 def test_entry_assertions_and_error_codes(mods):
     hip, v4, st, ao = mods
     q = torch.zeros(1, 2, 2048, 128, dtype=torch.bfloat16, device="cuda")
