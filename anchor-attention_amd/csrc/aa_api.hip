@@ -272,9 +272,6 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
-#ifdef AA_CLOCKS  // timing experiments only
-  a.L_out = const_cast<float*>(L);
-#endif
   return check_launch(run_flash(a, 1, (hipStream_t)stream), who);
 }
 

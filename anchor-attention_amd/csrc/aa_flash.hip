@@ -43,10 +43,7 @@ constexpr int kBN = 64;        // keys per LDS tile
 constexpr int kRowBytes = 256;   // one K/V row in LDS (128 bf16, unpadded, chunks swizzled)
 constexpr int kTileBytes = kBN * kRowBytes;
 constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
-#ifndef AA_DIST
-#define AA_DIST 4
-#endif
-constexpr int kDist = AA_DIST;    // MFMA operands are fetched from LDS this many MFMAs ahead of their use
+constexpr int kDist = 4;         // MFMA operands are fetched from LDS this many MFMAs ahead of their use
 constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
@@ -67,9 +64,6 @@ struct FlashSmem {
     __bf16 os[4][32 * kOsStride];  // epilogue staging, reuses the tile space
   };
   int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
-#ifdef AA_ONE_WG
-  char pad_one_wg[24576];
-#endif
 };
 
 __device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale, const bool bf16_chain) {
@@ -151,12 +145,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const int wr0 = R0 + wave * 32;
   const int my_row = wr0 + c32;
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
-#ifdef AA_CLOCKS  // timing experiments only: shader-clock and 100 MHz reference stamps
-#ifndef AA_CLOCKS_QBLK
-#define AA_CLOCKS_QBLK (n_qblk / 2)
-#endif
-  const long long aa_c0 = clock64(), aa_w0 = wall_clock64();
-#endif
 
   const __bf16* qp = p.q + b * p.q_sb + hq * p.q_sh;
   const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
@@ -270,13 +258,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     for (int m = 0; m < 4; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
   }
 
-#ifdef AA_CLOCKS
-  long long aa_ph[6] = {0, 0, 0, 0, 0, 0};
-  long long aa_t = clock64();
-#define AA_STAMP(i) { const long long t_ = clock64(); aa_ph[i] += t_ - aa_t; aa_t = t_; }
-#else
-#define AA_STAMP(i)
-#endif
 
   // key (or list position) that accumulator register r of 32-key half kb of the tile at key0 stands for
 #define AA_KEY_OF(kb, r) (key0 + 32 * (kb) + 8 * ((r) >> 2) + 4 * half + ((r) & 3))
@@ -330,7 +311,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   int32_t buf_step = kTileBytes;  // what takes the read addresses to the other LDS buffer
   for (int i = 0; i < n_tiles; ++i) {
     const int buf = i & 1;
-    AA_STAMP(5)
     const int key0 = AA_TILE_KEY0(i);
     if (MODE == kSparse && i + 1 < n_tiles && ((i + 1) & (kIdxWin / kBN - 1)) == 0) {
       // tile i+1 opens the next window; everyone finished reading the old one before the last barrier
@@ -343,15 +323,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // (the last tile fetches itself once more into the idle buffer, which keeps the instruction stream free of branches)
     const int i_next = i + 1 < n_tiles ? i + 1 : i;
     const int key0_next = AA_TILE_KEY0(i_next);
-#ifdef AA_NO_FETCH  // timing experiment: tiles after the first are not fetched (results are meaningless)
-#define AA_FETCH_ONE(n)
-#else
 #define AA_FETCH_ONE(n)                                                                                               \
   tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,   \
                                   lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes, k_voff, v_voff);
-#endif
-
-    AA_STAMP(0)
     // (a wave whose rows all lie above this tile - two of the four waves on the last tile of a causal work-group -
     // runs it fully masked: it would only wait at the barrier for the others anyway)
     {
@@ -386,7 +360,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         AA_FETCH_ONE(n)
         AA_FENCE;
       }
-      AA_STAMP(1)
 
       // ---- phase B: S1^T = K1 Q^T, with the soft-max of S0 between the MFMAs ---------------------
 #pragma unroll
@@ -431,7 +404,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         AA_S_MFMA(s1, n);
         AA_FENCE;
       }
-      AA_STAMP(2)
 
       // ---- phase C: O^T += V0^T P0^T, with the soft-max of S1 between the MFMAs --------------------
 #pragma unroll
@@ -491,7 +463,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
 #undef AA_OPERAND_FETCH
 #undef AA_S_MFMA
-      AA_STAMP(3)
 #undef AA_K_FETCH
     }
 #undef AA_FETCH_ONE
@@ -504,7 +475,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     buf_step = -buf_step;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
     __syncthreads();
-    AA_STAMP(4)
   }
 #undef AA_TILE_KEY0
 #undef AA_KEY_OF
@@ -516,14 +486,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #undef AA_PV_MFMA
 #undef AA_FENCE
 
-#ifdef AA_CLOCKS
-  if (MODE != kDense && tid == 0 && qblk == AA_CLOCKS_QBLK && hq == 0 && b == 0) {
-    p.L_out[bh * p.n_ctx + p.n_ctx - 1] = (float)(clock64() - aa_c0);
-    p.L_out[bh * p.n_ctx + p.n_ctx - 2] = (float)(wall_clock64() - aa_w0);
-    p.L_out[bh * p.n_ctx + p.n_ctx - 3] = (float)n_tiles;
-    for (int i = 0; i < 6; ++i) p.L_out[bh * p.n_ctx + p.n_ctx - 4 - i] = (float)aa_ph[i];
-  }
-#endif
   // ---- epilogue --------------------------------------------------------------------------------
   const float l_tot = l_run + xor32(l_run);
   if (MODE == kAnchor) {
