@@ -97,12 +97,13 @@ def make_inputs(name, seed, qbar_mode, device):
 
 def cpu_baseline():
     """The CPU oracle (our numpy restatement of the reference algorithm - the reference has no CPU
-    path of its own) timed on this host on a bounded sample: the config-0 shape (N=4096, 32/8 heads)."""
+    path of its own) timed on this host on a bounded sample of the workload: one layer of the same head
+    configuration at N=16384 (10-30 s of CPU work; the full 128k layer would take tens of minutes)."""
     import numpy as np
     from anchor_attn.synthetic import make_qkv
     from oracle import anchor_oracle as ao
-    n_ctx, hq, hkv = 4096, 32, 8
-    q, k, v, _ = make_qkv(n_ctx, hq, hkv, n_stripes=64, seed=0)
+    n_ctx, hq, hkv = 16384, 32, 8
+    q, k, v, _ = make_qkv(n_ctx, hq, hkv, n_stripes=256, seed=0)
     Q, K, V = (t.float().numpy() for t in (q, k, v))
     t0 = time.time()
     res = ao.anchor_attn_reference(Q, K, V, difference=12.0)
