@@ -518,3 +518,32 @@ def test_maximum_context_one_million_tokens(mods):
     with pytest.raises(hip.AnchorAttnHipError):
         too_long = torch.empty(1, 1, N + S, D, dtype=torch.bfloat16, device="cuda")
         v4.anchor_attn(too_long, too_long, too_long)
+
+
+def test_gpu_matches_committed_fixture(mods):
+    """The kernels against the committed fixture of tests/golden/ (oracle results for a seeded case; no oracle
+    call at test time): counts and index lists, and the sampled rows of M, L and the output."""
+    import importlib.util
+    import os
+    hip, v4, st, ao = mods
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_oracle_fixture", os.path.join(here, "make_oracle_fixture.py"))
+    fx = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(fx)
+    want = np.load(os.path.join(here, "oracle_small_case.npz"))
+    from anchor_attn.synthetic import make_qkv
+    q, k, v, _ = make_qkv(**fx.CASE)
+    q, k, v = q.cuda(), k.cuda(), v.cuda()
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(q, k, M, BS, STEP, fx.THETA * LOG2E, B, H, N, D, SM)
+    out, ratio = v4.anchor_attn(q, k, v, difference=fx.THETA)
+    got, got_counts = _packed_lists(hip, coords, counts, N)
+    flat = np.concatenate([got[0][h][bb] for h in range(H) for bb in range(N // S)])
+    assert np.setxor1d(flat, want["coords"]).size <= 2 and abs(int(got_counts.sum()) - int(want["counts"].sum())) <= 2
+    rows = torch.from_numpy(fx.ROWS).cuda()
+    np.testing.assert_allclose(M[0][:, rows].cpu().numpy(), want["M"], atol=3e-4)
+    np.testing.assert_allclose(L[0][:, rows].cpu().numpy(), want["L"], rtol=1e-3)
+    err = np.abs(out[0][:, rows].float().cpu().numpy() - want["out"])
+    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    assert abs(float(ratio) - float(want["ratio"])) < 1e-4

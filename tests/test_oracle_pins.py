@@ -309,3 +309,22 @@ def test_intended_geometry_candidate_range_and_dense_limit():
     assert np.abs(res.out - dense).max() < 2e-2 and np.abs(res.out - dense).mean() < 2e-3
     as_run = ao.anchor_attn_reference(Q, K, V, difference=1e4)
     assert np.abs(as_run.out[0, 0, 2 * 2048:] - dense[0, 0, 2 * 2048:]).max() > 5e-2
+
+
+def test_oracle_regression_fixture():
+    """The committed fixture (tests/golden/, written by this repository's oracle, see the script there) still
+    matches: index lists exactly, floating-point results to BLAS-rounding tolerance."""
+    import importlib.util
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_oracle_fixture", os.path.join(here, "make_oracle_fixture.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    got = mod.run_case()
+    want = np.load(os.path.join(here, "oracle_small_case.npz"))
+    assert np.array_equal(got["stripe_positions"], want["stripe_positions"])
+    assert np.array_equal(got["counts"], want["counts"]) and np.array_equal(got["coords"], want["coords"])
+    assert float(got["ratio"]) == float(want["ratio"])
+    np.testing.assert_allclose(got["M"], want["M"], atol=1e-5)
+    np.testing.assert_allclose(got["L"], want["L"], rtol=1e-5)
+    np.testing.assert_allclose(got["out"], want["out"], atol=1e-5)
