@@ -17,9 +17,13 @@ Parity status: the reference ships no golden vectors for this path, so every fun
 is pinned by mathematics instead (tests/test_oracle_*.py): float64 brute force over the
 explicit key sets, library softmax attention where the key set is the full causal prefix,
 closed forms for theta -> +/- infinity, an independent bf16 rounding (torch's cast) and the
-multiplicity formula for double-counted keys.  Not pinned by anything but reading of the
-compiler's promotion rules: the bf16 scale chain of stage 1 (``q1_scale_chain``), which is
-therefore a switch (``stage1_scale_mode``) - "parity unpinned" for that one choice.
+multiplicity formula for double-counted keys.  The two query pre-scaling chains
+(``q1_scale_chain``: bf16 products for stage 1, whose kernel takes ``sm_scale`` as a constexpr;
+``q3_scale_chain``: float32 products for stage 3, whose kernel takes it at run time) are pinned
+bit for bit against the Triton toolchain itself: tests/triton_promotion_probe.py compiles the two
+forms of the reference's expression as micro-kernels of its own, and its outputs on an MI355X are
+the fixture tests/golden/triton_scale_chain_probe.npz (Triton 3.6.0; the reference pins no Triton
+version).  ``stage1_scale_mode`` remains a switch.
 
 Conventions: ``Q`` is ``[B, Hq, N, D]``, ``K``/``V`` are ``[B, Hkv, N, D]`` with ``Hkv | Hq``
 (query head ``h`` reads KV head ``h // (Hq // Hkv)``, the order ``repeat_kv`` produces);

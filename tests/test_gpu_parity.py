@@ -547,3 +547,33 @@ def test_gpu_matches_committed_fixture(mods):
     err = np.abs(out[0][:, rows].float().cpu().numpy() - want["out"])
     assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
     assert abs(float(ratio) - float(want["ratio"])) < 1e-4
+
+
+def test_triton_promotion_rule_live(mods, tmp_path):
+    """The same probe compiled and run here (skipped when Triton is not installed): over every finite bf16 value,
+    the constexpr form equals the oracle's bf16 chain and the run-time form its float32 chain, bit for bit."""
+    pytest.importorskip("triton")
+    import os
+    import subprocess
+    import sys
+    hip, v4, st, ao = mods
+    out = tmp_path / "probe.npz"
+    probe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "triton_promotion_probe.py")
+    subprocess.run([sys.executable, probe, str(out), "cuda"], check=True, timeout=170)
+    r = np.load(out)
+    x = r["x"]
+    for name in ("d128", "d64", "odd"):
+        sm = float(r[f"sm_{name}"])
+        assert np.array_equal(r[f"constexpr_{name}"], ao.q1_scale_chain(x, sm, mode="bf16_chain"))
+        assert np.array_equal(r[f"runtime_{name}"], ao.q3_scale_chain(x, sm))
+    raw = (r["s2_dot"] * np.float32(float(r["s2_sm"]) * ao.LOG2E)).astype(np.float32)
+    assert np.array_equal(ao.rn16(raw), r["s2_qk"])
+    hit = (ao.rn16(raw) + np.float32(float(r["s2_theta"]) * ao.LOG2E)) >= r["s2_anchor"]
+    assert np.array_equal(hit, r["s2_hit"].astype(bool))
+    # pooling: float32 anchors pool to the same bf16 values; bf16 queries do not - this Triton release reduces
+    # them in bf16, the oracle (and the library) in float32, which is the closer of the two to the exact mean
+    exact = r["pool_q"].reshape(8, 16, 128, 128).astype(np.float64).mean(axis=2)
+    ours = np.stack([ao.pooled_queries(r["pool_q"][i], 128) for i in range(8)])
+    for i in range(8):
+        assert np.array_equal(ao.pooled_anchors(r["pool_m"][i], 128)[0], r["pool_abar"][i])
+    assert np.abs(ours - exact).max() <= np.abs(r["pool_qbar"] - exact).max() <= 0.02

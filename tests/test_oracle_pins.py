@@ -328,3 +328,36 @@ def test_oracle_regression_fixture():
     np.testing.assert_allclose(got["M"], want["M"], atol=1e-5)
     np.testing.assert_allclose(got["L"], want["L"], rtol=1e-5)
     np.testing.assert_allclose(got["out"], want["out"], atol=1e-5)
+
+
+def test_scale_chains_match_triton_compiled_outputs():
+    """Pins the two query pre-scaling chains against the Triton toolchain itself.  tests/golden/
+    triton_scale_chain_probe.npz holds what tests/triton_promotion_probe.py (own micro-kernels with the two forms
+    of the reference's expression, compiled by Triton 3.6.0 for gfx950 and run on an MI355X) returned for every
+    bf16 value with 2^-8 <= |x| < 2^8 and for zero: a constexpr sm_scale keeps the products in bf16 (stage 1), a
+    run-time sm_scale promotes them to float32 (stage 3).  Bit-exact, three scales."""
+    import os
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "triton_scale_chain_probe.npz"))
+    unbits = lambda b: (b.astype(np.uint32) << 16).view(np.float32)
+    x = unbits(fx["x_bf16_bits"])
+    assert x.size > 4000
+    for name in ("d128", "d64", "odd"):
+        sm = float(fx[f"sm_{name}"])
+        want1, want3 = unbits(fx[f"constexpr_{name}_bf16_bits"]), unbits(fx[f"runtime_{name}_bf16_bits"])
+        assert np.array_equal(ao.q1_scale_chain(x, sm, mode="bf16_chain"), want1)
+        assert np.array_equal(ao.q3_scale_chain(x, sm), want3)
+        assert np.array_equal(ao.q1_scale_chain(x, sm, mode="fp32"), want3)
+        assert (want1 != want3).sum() > 500  # the two chains are different functions, so the pin discriminates
+    # element-wise stage-2 test: constexpr qk_scale * literal, bf16 rounding of the score, float32 "+ diff >= anchor"
+    dot, anchor = fx["s2_dot"], unbits(fx["s2_anchor_bf16_bits"])
+    sm, theta = float(fx["s2_sm"]), float(fx["s2_theta"])
+    raw = (dot * np.float32(sm * ao.LOG2E)).astype(np.float32)
+    assert np.array_equal(ao.rn16(raw), unbits(fx["s2_qk_bf16_bits"]))
+    hit = (ao.rn16(raw) + np.float32(theta * ao.LOG2E)) >= anchor
+    assert np.array_equal(hit, fx["s2_hit"].astype(bool)) and 0.2 < hit.mean() < 0.8
+    assert ((raw + np.float32(theta * ao.LOG2E) >= anchor) != hit).sum() > 300       # un-rounded score: a different test
+    # the oracle's own boundary helper agrees with the compiled decisions
+    for i in range(0, dot.size, 97):
+        xb = ao.stage2_decision_boundary(float(anchor[i]), theta)
+        if float(raw[i]) != xb:  # (exactly on the midpoint the bf16 tie rule decides)
+            assert (float(raw[i]) > xb) == bool(fx["s2_hit"][i])
