@@ -577,3 +577,19 @@ def test_triton_promotion_rule_live(mods, tmp_path):
     for i in range(8):
         assert np.array_equal(ao.pooled_anchors(r["pool_m"][i], 128)[0], r["pool_abar"][i])
     assert np.abs(ours - exact).max() <= np.abs(r["pool_qbar"] - exact).max() <= 0.02
+
+
+def test_integration_stub_runs_as_written(mods, llama_small, repo_root):
+    """The ctypes stub printed in INTEGRATION.md, executed verbatim (only the library path is filled in), gives
+    the same output and ratio as the package's own host layer."""
+    import re
+    hip, v4, st, ao = mods
+    text = open(str(repo_root) + "/INTEGRATION.md").read()
+    block = re.search(r"## 2\..*?```python\n(.*?)```", text, re.S).group(1)
+    block = block.replace('"libanchor_attn_hip.so"', repr(hip.library_path()))
+    ns = {}
+    exec(compile(block, "INTEGRATION.md", "exec"), ns)
+    (q, k, v), _, _ = llama_small
+    out, ratio = ns["anchor_attn_mi355x"](q, k, v)
+    want, want_ratio = v4.anchor_attn(q, k, v)
+    assert torch.equal(out, want) and abs(float(ratio) - float(want_ratio)) < 1e-9
