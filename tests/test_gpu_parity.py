@@ -252,6 +252,20 @@ def test_single_big_block_is_plain_causal_attention(mods):
     assert err.max() < 3e-2 and err.mean() < 2e-3
 
 
+@pytest.mark.parametrize("n_bb,hq,hkv,step,theta,seed,base,dist", [
+    (2, 1, 1, 16, 8.0, 101, 5e5, "uniform"),
+    (5, 2, 2, 16, 15.5, 102, 1e4, "powerlaw"),
+    (3, 8, 1, 16, 12.0, 103, 1e6, "uniform"),
+    (2, 3, 3, 32, 13.0, 104, 5e5, "powerlaw"),
+    (4, 6, 2, 16, 10.5, 105, 5e5, "uniform"),
+    (3, 2, 1, 32, 16.0, 106, 1e6, "uniform"),
+])
+def test_assorted_shapes_and_thresholds(mods, n_bb, hq, hkv, step, theta, seed, base, dist):
+    """Head groupings 1:1 to 8:1, both step sizes, thresholds from 8 to 16, three RoPE bases, both stripe laws."""
+    q, k, v, _ = _case(n_bb * BS * step, hq, hkv, 40 * n_bb, seed=seed, rope_base=base, stripe_dist=dist)
+    _end_to_end(mods, q, k, v, theta, max_excused=8, step=step)
+
+
 def test_theta_minus_inf_two_big_blocks_equals_library_attention(mods):
     hip, v4, st, ao = mods
     q, k, v, _ = _case(2 * S, 4, 2, 32, seed=5)
