@@ -117,10 +117,16 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   __shared__ __attribute__((aligned(16))) __bf16 a_lds[2][32 * kARowStride];
   __shared__ __attribute__((aligned(16))) float thr_lds[2][32];
 
-  const int T = blockIdx.x;  // key super-tile (kTilesPerWg * 128 keys)
-  const int kvh = blockIdx.y, b = blockIdx.z;
+  // Work-groups are renumbered so that each XCD owns a contiguous range ordered (batch, KV head, super-tile): the
+  // pooled queries a work-group streams are those of its KV head's query heads (1 MiB per KV head at 128k tokens),
+  // which then stay in that XCD's L2 instead of every XCD cycling through all heads' pooled queries.
   const int n_bb = p.n_ctx / p.big_block;
   const int n_t = p.n_ctx / 128;
+  const int n_super = n_t / kTilesPerWg;
+  uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+  const int T = vid % n_super;  // key super-tile (kTilesPerWg * 128 keys); ascending = heaviest first
+  vid /= n_super;
+  const int kvh = vid % p.n_kv_heads, b = vid / p.n_kv_heads;
   const int n_pr = n_t;  // pooled rows per head (block_size == 128)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -245,7 +251,7 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
 
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
   const int step = a.big_block / a.block_size;
-  const dim3 grid(a.n_ctx / (128 * kKB), a.n_kv_heads, a.batch);
+  const dim3 grid((uint32_t)(a.n_ctx / (128 * kKB)) * a.n_kv_heads * a.batch);
   if (step == 16) hipLaunchKernelGGL(select_scores_kernel<16>, grid, dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(select_scores_kernel<32>, grid, dim3(256), 0, stream, a);
   return hipGetLastError();
