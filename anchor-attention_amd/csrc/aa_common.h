@@ -52,11 +52,24 @@ __host__ __device__ inline int64_t coords_tri(int64_t bb, int64_t S, int64_t bs)
   return bb <= 1 ? 0 : S * (bb - 1) * bb / 2 - 2 * bs * (bb - 1);
 }
 
-// XCD-aware work-group renumbering: consecutive hardware work-group ids go round-robin over the
-// 8 XCDs (each with its own L2); give every XCD one contiguous range of logical ids so that
-// neighbours in the logical order (which share K/V tiles) hit the same L2.
-__device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t total) {
-  return (total % 8u == 0u) ? (wg % 8u) * (total / 8u) + wg / 8u : wg;
+// XCD-aware work-group renumbering.  Consecutive hardware work-group ids go round-robin over the 8 XCDs (each
+// with its own L2).  The work consists of `n_units` units (a KV head of one batch element) of `per_unit`
+// work-groups each, ordered heaviest first inside a unit; work-groups of one unit read the same K/V rows or pooled
+// queries.  Returns the logical index unit * per_unit + idx such that
+//   n_units % 8 == 0 : every XCD owns n_units / 8 whole units, in order;
+//   8 % n_units == 0 : s = 8 / n_units XCDs share a unit and take its rows alternately (row = idx / inner, the
+//                      `inner` work-groups of a row stay together), so that each gets the same mix of heavy and light;
+//   otherwise        : the hardware order is kept.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t wg, uint32_t n_units, uint32_t per_unit, uint32_t inner) {
+  const uint32_t total = n_units * per_unit;
+  const uint32_t xcd = wg % 8u, k = wg / 8u;
+  if (total % 8u != 0u) return wg;
+  if (n_units % 8u == 0u) return xcd * (total / 8u) + k;
+  if (8u % n_units == 0u) {
+    const uint32_t s = 8u / n_units;
+    if ((per_unit / inner) % s == 0u) return (xcd / s) * per_unit + ((k / inner) * s + xcd % s) * inner + k % inner;
+  }
+  return wg;
 }
 
 // ---- error plumbing (host) -------------------------------------------------------------------

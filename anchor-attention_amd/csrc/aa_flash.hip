@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   // ---- which rows ----------------------------------------------------------------------------
   const int group = p.n_q_heads / p.n_kv_heads;
   const int n_qblk = p.n_ctx / BM;
-  uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qblk, group);
   const int g = vid % group;  vid /= group;
   int qblk = vid % n_qblk;    vid /= n_qblk;
   const int kvh = vid % p.n_kv_heads;

@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   const int n_bb = p.n_ctx / p.big_block;
   const int n_t = p.n_ctx / 128;
   const int n_super = n_t / kTilesPerWg;
-  uint32_t vid = xcd_remap(blockIdx.x, gridDim.x);
+  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, n_super, 1);
   const int T = vid % n_super;  // key super-tile (kTilesPerWg * 128 keys); ascending = heaviest first
   vid /= n_super;
   const int kvh = vid % p.n_kv_heads, b = vid / p.n_kv_heads;
