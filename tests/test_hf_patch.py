@@ -111,3 +111,33 @@ def test_patched_model_equals_dense_model_when_the_window_covers_everything():
     assert torch.isfinite(b).all()
     assert (a - b).abs().max() < 0.08 * a.abs().max()
     assert (a - b).abs().mean() < 0.01 * a.abs().mean() + 1e-3
+
+
+@pytest.mark.gpu
+def test_patched_qwen2_model():
+    """The same plug under Qwen2 (attention biases, its own config class): window-covers-everything equality with
+    the dense model, and a real sparse prefill that stays finite and reports a ratio."""
+    from transformers import Qwen2Config, Qwen2ForCausalLM
+
+    from anchor_attn import patch_model
+    from anchor_attn.src.modules.qwen2 import anchor_attention as plug
+    torch.manual_seed(0)
+    cfg = Qwen2Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, vocab_size=1000, max_position_embeddings=16384, rope_theta=1e6)
+    assert cfg.hidden_size // cfg.num_attention_heads == 128
+    ref = Qwen2ForCausalLM(cfg).eval().to(torch.bfloat16).cuda()
+    m = Qwen2ForCausalLM(cfg).eval().to(torch.bfloat16).cuda()
+    m.load_state_dict(ref.state_dict())
+    patch_model(m, "anchor_attn", {"theta": -1e4})
+    x = torch.randint(0, 1000, (1, 2 * 2048 + 5), device="cuda")
+    with torch.no_grad():
+        a = ref(x, logits_to_keep=32).logits.float()
+        b = m(x, logits_to_keep=32).logits.float()
+    assert torch.isfinite(b).all() and (a - b).abs().max() < 0.08 * a.abs().max()
+    patch_model(m, "anchor_attn", {"theta": 12})
+    y = torch.randint(0, 1000, (1, 3 * 2048), device="cuda")
+    with torch.no_grad():
+        c = m(y, logits_to_keep=1).logits
+    import anchor_attn.src.modules.llama.anchor_attention as llama_plug
+    assert torch.isfinite(c).all() and plug.anchor_attention_forward is llama_plug.anchor_attention_forward
+    assert 0 < float(llama_plug.last_ratio) <= 1.0
