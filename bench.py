@@ -162,7 +162,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the operator is embarrassingly parallel over KV-head "
-                 "groups; see DESIGN.md for how it would shard) - run with --gpus 1")
+                 "groups, which would shard across GPUs with no exchange) - run with --gpus 1")
 
     import torch
     from anchor_attn.src.ops import _hip, anchor_attn_v4 as v4, anchor_step_1_2_v2 as st

@@ -594,7 +594,7 @@ def test_triton_promotion_rule_live(mods, tmp_path):
 
 
 def test_integration_stub_runs_as_written(mods, llama_small, repo_root):
-    """The ctypes stub printed in INTEGRATION.md, executed verbatim (only the library path is filled in), gives
+    """The ctypes stub printed in the integration guide, executed verbatim (only the library path is filled in), gives
     the same output and ratio as the package's own host layer."""
     import re
     hip, v4, st, ao = mods
@@ -602,7 +602,7 @@ def test_integration_stub_runs_as_written(mods, llama_small, repo_root):
     block = re.search(r"## 2\..*?```python\n(.*?)```", text, re.S).group(1)
     block = block.replace('"libanchor_attn_hip.so"', repr(hip.library_path()))
     ns = {}
-    exec(compile(block, "INTEGRATION.md", "exec"), ns)
+    exec(compile(block, "integration-guide-stub", "exec"), ns)
     (q, k, v), _, _ = llama_small
     out, ratio = ns["anchor_attn_mi355x"](q, k, v)
     want, want_ratio = v4.anchor_attn(q, k, v)
