@@ -19,11 +19,17 @@ from typing import Optional, Tuple
 import torch
 import torch.nn.functional as F
 
-from anchor_attn.src.ops.anchor_attn_v4 import anchor_attn
+from anchor_attn.src.ops.anchor_attn_v4 import LOG2E, _anchor_attn, anchor_attn, dense_causal_attention
 
 ATTN_NAME = "anchor_attn"
+DENSE_ATTN_NAME = "anchor_attn_dense"
 
-# sparsity ratio of the most recent prefill call (0-dim device tensor), for measurement scripts
+# Measurement scripts set ``record_ratio``; the plug then also asks the operator for the per-big-block counts and
+# leaves the sparsity ratio of the most recent prefill call in ``last_ratio`` as a 0-dim DEVICE tensor (nothing is
+# copied to the host and nothing is logged, so the model stays free of host synchronisation either way).  By default
+# the operator is called with ``return_computational_ratio=False`` as the reference's caller does
+# (modules/llama/anchor_attention.py:92-100).
+record_ratio: bool = False
 last_ratio: Optional[torch.Tensor] = None
 
 
@@ -56,10 +62,37 @@ def anchor_attention_forward(module, query: torch.Tensor, key: torch.Tensor, val
         return out, None
     pad = N % big
     main = N - pad
-    res = anchor_attn(query[:, :, :main], key[:, :, :main], value[:, :, :main], sm_scale=scaling,
-                      block_size=block_size, step=step, difference=theta,
-                      return_computational_ratio=True, out=out_bhnd[:, :, :main])
-    last_ratio = res[1]
+    if record_ratio:
+        sm_scale = scaling if scaling else 1.0 / (D ** 0.5)
+        _, last_ratio = _anchor_attn(query[:, :, :main], key[:, :, :main], value[:, :, :main], sm_scale, block_size, step,
+                                     theta * LOG2E, True, out=out_bhnd[:, :, :main])
+    else:
+        anchor_attn(query[:, :, :main], key[:, :, :main], value[:, :, :main], sm_scale=scaling,
+                    block_size=block_size, step=step, difference=theta,
+                    return_computational_ratio=False, out=out_bhnd[:, :, :main])
     if pad:
+        out_bhnd[:, :, main:].copy_(_dense(query[:, :, main:], key, value, None, scaling, main))
+    return out, None
+
+
+def dense_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                            attention_mask: Optional[torch.Tensor], dropout: float = 0.0,
+                            scaling: Optional[float] = None, **kwargs) -> Tuple[torch.Tensor, None]:
+    """Plain causal attention on the library's own MFMA core (``aa_dense_causal_fwd``): the dense baseline "built on
+    the same kernels" that the sparse operator is compared with.  Counterpart of the reference's ``"flash"`` pattern
+    (modules/patch.py:128-130 -> modules/llama/flash_attention.py, ops/flash_attn_triton.py:641-657), with the same
+    division of labour as the sparse plug: a fresh unpadded bf16 prefill goes through the kernel in multiples of
+    128 rows, the remaining tail rows, decode steps and padded batches through the framework's dense attention."""
+    B, Hq, N, D = query.shape
+    n_kv = key.shape[2]
+    out = torch.empty(B, N, Hq, D, dtype=query.dtype, device=query.device)
+    out_bhnd = out.transpose(1, 2)
+    kernel_ok = N >= 128 and n_kv == N and attention_mask is None and query.dtype == torch.bfloat16 and query.is_cuda
+    if not kernel_ok:
+        out_bhnd.copy_(_dense(query, key, value, attention_mask, scaling, n_kv - N if attention_mask is None else None))
+        return out, None
+    main = N - N % 128
+    dense_causal_attention(query[:, :, :main], key[:, :, :main], value[:, :, :main], sm_scale=scaling, out=out_bhnd[:, :, :main])
+    if main < N:
         out_bhnd[:, :, main:].copy_(_dense(query[:, :, main:], key, value, None, scaling, main))
     return out, None

@@ -1,8 +1,11 @@
 """``patch_model``: switch a Hugging Face causal LM to AnchorAttention prefill.
 
 Counterpart of the reference's anchor_attn/src/modules/patch.py:116-164,290-327 for the patterns on the
-AnchorAttention path ("default", "flash", "anchor_attn"); the competitor patterns of the reference are not
-part of this package and raise ``ValueError``.  In transformers 5 the attention product is selected by
+AnchorAttention path: "default", "flash" (the framework's library attention), "dense" (plain causal attention
+on this package's own MFMA kernel - the baseline "built on the same kernels"), "anchor_attn" and
+"anchor_attn_lite" (in the reference the two names select the same forward with the same defaults,
+patch.py:36-45,142-144); the competitor patterns of the reference are not part of this package and raise
+``ValueError``.  In transformers 5 the attention product is selected by
 name through ``AttentionInterface``, so patching is: register the plug once, point the model's config at it,
 and copy the pattern's parameters onto the config (patch.py:106-109 does the same ``setattr`` loop).
 """
@@ -13,10 +16,13 @@ from my_utils import Logger
 ATTENTION_CONFIG_EXAMPLE = {
     "default": {},
     "flash": {},
+    "dense": {},
     "anchor_attn": {"block_size_M": 128, "theta": 12, "step": 16},
+    "anchor_attn_lite": {"block_size_M": 128, "theta": 12, "step": 16},
 }
 
 _SUPPORTED_MODELS = ("llama", "qwen2")
+SUPPORTED_BLOCK_SIZES = (128,)
 
 
 def get_config_example(pattern: str = None):
@@ -29,19 +35,22 @@ def _register():
     from transformers import AttentionInterface, AttentionMaskInterface
     from transformers.masking_utils import sdpa_mask
 
-    from anchor_attn.src.modules.llama.anchor_attention import ATTN_NAME, anchor_attention_forward
-    if ATTN_NAME not in AttentionInterface().valid_keys():
-        AttentionInterface.register(ATTN_NAME, anchor_attention_forward)
-        # same mask convention as SDPA: None when the mask is purely causal, a boolean mask otherwise
-        AttentionMaskInterface.register(ATTN_NAME, sdpa_mask)
-    return ATTN_NAME
+    from anchor_attn.src.modules.llama.anchor_attention import (ATTN_NAME, DENSE_ATTN_NAME, anchor_attention_forward,
+                                                                dense_attention_forward)
+    for name, fn in ((ATTN_NAME, anchor_attention_forward), (DENSE_ATTN_NAME, dense_attention_forward)):
+        if name not in AttentionInterface().valid_keys():
+            AttentionInterface.register(name, fn)
+            # same mask convention as SDPA: None when the mask is purely causal, a boolean mask otherwise
+            AttentionMaskInterface.register(name, sdpa_mask)
+    return ATTN_NAME, DENSE_ATTN_NAME
 
 
 def patch_model(model, pattern: str, config: dict = None):
     """Patch ``model`` (a transformers ``PreTrainedModel`` of the Llama or Qwen2 family) in place.
 
-    pattern: "default" (leave as is), "flash" (library dense attention) or "anchor_attn".
-    config : for "anchor_attn" ``{"block_size_M": 128, "theta": 12, "step": 16}`` (the defaults).
+    pattern: "default" (leave as is), "flash" (the framework's library attention), "dense" (causal attention on this
+             package's own kernel), "anchor_attn" or "anchor_attn_lite" (same operator, same defaults).
+    config : for the anchor patterns ``{"block_size_M": 128, "theta": 12, "step": 16}`` (the defaults).
     """
     from transformers import PreTrainedModel
     if not isinstance(model, PreTrainedModel):
@@ -57,10 +66,12 @@ def patch_model(model, pattern: str, config: dict = None):
     cfg.update(config or {})
     if pattern == "flash":
         model.set_attn_implementation("sdpa")
+    elif pattern == "dense":
+        model.set_attn_implementation(_register()[1])
     else:
-        if cfg["step"] not in (16, 32) or cfg["block_size_M"] != 128:
-            raise ValueError("anchor_attn supports block_size_M = 128 and step in (16, 32)")
-        model.set_attn_implementation(_register())
+        if cfg["step"] not in (16, 32) or cfg["block_size_M"] not in SUPPORTED_BLOCK_SIZES:
+            raise ValueError(f"{pattern} supports block_size_M in {SUPPORTED_BLOCK_SIZES} and step in (16, 32)")
+        model.set_attn_implementation(_register()[0])
         for k, v in cfg.items():
             setattr(model.config, k, v)
     Logger.log(f"replace attention with {pattern}: {cfg}")

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _LIB_NAME = "libanchor_attn_hip.so"
 _lib = None
@@ -37,9 +37,9 @@ _SIGNATURES = {
     "aa_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "aa_stage1_anchor_fwd": (c_int, _T3 * 3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_float, c_int, c_void_p]),
     "aa_pool_q_anchor": (c_int, _T3 + [c_void_p] * 3 + [c_int, c_int, c_int, c_int, c_int, c_void_p]),
-    "aa_stage2_select": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_float, c_float, c_int, c_void_p]),
+    "aa_stage2_select": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_void_p]),
     "aa_stage3_sparse_fwd": (c_int, _T3 * 3 + [c_void_p] * 5 + _T3 + _DIMS5 + [c_int, c_int, c_float, c_void_p]),
-    "aa_anchor_attn_fwd": (c_int, _T3 * 4 + [c_void_p, c_size_t, c_void_p] + _DIMS5 + [c_int, c_int, c_float, c_float, c_int, c_int, c_void_p]),
+    "aa_anchor_attn_fwd": (c_int, _T3 * 4 + [c_void_p, c_size_t, c_void_p] + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_int, c_void_p]),
     "aa_dense_causal_fwd": (c_int, _T3 * 4 + _DIMS5 + [c_float, c_void_p]),
 }
 

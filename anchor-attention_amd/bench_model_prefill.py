@@ -2,7 +2,9 @@
 
 BASELINE config 4: the 32-layer Llama-3.1-8B architecture (hidden 4096, FFN 14336, 32/8 heads, vocab 128256,
 RoPE base 5e5) with random-init bf16 weights and random token ids at N = 131072 on one GPU; reports the
-prefill time with the operator, its attention share, and the same model on the library's dense attention.
+prefill time with the operator and its attention share, and the same model with dense attention twice: on this
+package's own MFMA kernel (pattern "dense", the baseline "built on the same kernels") and on the framework's
+library attention (pattern "flash").
 There is no checkpoint or dataset involved: weights and tokens are synthetic, so the sparsity a trained
 model would show is not reproduced - the numbers are timings of the code path, and say so.
 
@@ -24,7 +26,7 @@ def main():
     ap.add_argument("--n-ctx", type=int, default=131072)
     ap.add_argument("--theta", type=float, default=12.0)
     ap.add_argument("--reps", type=int, default=2)
-    ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention run of the same model")
+    ap.add_argument("--no-dense", action="store_true", help="skip the dense-attention runs of the same model")
     args = ap.parse_args()
 
     import torch
@@ -46,15 +48,17 @@ def main():
 
     # time spent inside the attention plug, by events around every call
     spans = []
-    inner = plug.anchor_attention_forward
+    plug.record_ratio = True  # the ratio stays a device tensor; it is read after the prefill has finished
 
-    def timed(*a, **k):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        r = inner(*a, **k)
-        e1.record()
-        spans.append((e0, e1, plug.last_ratio))
-        return r
+    def timed_plug(inner):
+        def timed(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = inner(*a, **k)
+            e1.record()
+            spans.append((e0, e1, plug.last_ratio if inner is plug.anchor_attention_forward else None))
+            return r
+        return timed
 
     def prefill(reps):
         best = None
@@ -75,17 +79,26 @@ def main():
 
     patch_model(model, "anchor_attn", {"theta": args.theta})
     from transformers import AttentionInterface
-    AttentionInterface.register(plug.ATTN_NAME, timed)
+    AttentionInterface.register(plug.ATTN_NAME, timed_plug(plug.anchor_attention_forward))
+    AttentionInterface.register(plug.DENSE_ATTN_NAME, timed_plug(plug.dense_attention_forward))
     ms, attn_ms, ratios, logits = prefill(args.reps)
     res = {"workload": f"llama3.1-8b architecture, {args.layers} layers, random-init bf16, N={args.n_ctx}, theta={args.theta}",
            "prefill_ms_anchor_attn": ms, "attention_ms": attn_ms, "attention_share": attn_ms / ms,
            "mean_sparsity_ratio": sum(ratios) / max(len(ratios), 1), "logits_finite": bool(torch.isfinite(logits).all())}
-    AttentionInterface.register(plug.ATTN_NAME, inner)
     if not args.no_dense:
+        patch_model(model, "dense")
+        dms, dattn, _, dlogits = prefill(1)
+        res["prefill_ms_dense_own_kernel"] = dms
+        res["attention_ms_dense_own_kernel"] = dattn
+        res["speedup_vs_dense_own_kernel"] = dms / ms
+        res["attention_speedup_vs_dense_own_kernel"] = dattn / attn_ms
         patch_model(model, "flash")
-        dms, _, _, _ = prefill(1)
-        res["prefill_ms_dense_sdpa"] = dms
-        res["speedup_vs_dense"] = dms / ms
+        fms, _, _, flogits = prefill(1)
+        res["prefill_ms_dense_library_sdpa"] = fms
+        res["speedup_vs_dense_library_sdpa"] = fms / ms
+        res["dense_own_vs_library_max_logit_diff"] = float((dlogits.float() - flogits.float()).abs().max())
+    AttentionInterface.register(plug.ATTN_NAME, plug.anchor_attention_forward)
+    AttentionInterface.register(plug.DENSE_ATTN_NAME, plug.dense_attention_forward)
     print(json.dumps(res))
 
 

@@ -26,7 +26,8 @@ struct Dims {
   int batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step;
 };
 
-int check_dims(const Dims& d, const char* who) {
+// Checks every entry point shares: head counts, head_dim, and the sizes one launch can address.
+int check_common_dims(const Dims& d, const char* who) {
   if (d.batch <= 0 || d.n_q_heads <= 0 || d.n_kv_heads <= 0 || d.n_ctx <= 0) {
     set_error("%s: batch, head counts and n_ctx must be positive (got %d, %d, %d, %d)", who, d.batch, d.n_q_heads, d.n_kv_heads, d.n_ctx);
     return AA_EBADARG;
@@ -39,6 +40,24 @@ int check_dims(const Dims& d, const char* who) {
     set_error("%s: head_dim %d is not supported (only 128)", who, d.head_dim);
     return AA_EUNSUPPORTED;
   }
+  if (d.n_ctx % 128 != 0) {
+    set_error("%s: n_ctx %d must be a multiple of 128", who, d.n_ctx);
+    return AA_EUNSUPPORTED;
+  }
+  if (d.n_ctx > (1 << 20)) {
+    set_error("%s: n_ctx %d is larger than 1048576", who, d.n_ctx);
+    return AA_EUNSUPPORTED;
+  }
+  if ((int64_t)d.batch * d.n_q_heads * (d.n_ctx / 128) > 0x7fffffffLL) {
+    set_error("%s: problem too large for one launch", who);
+    return AA_EUNSUPPORTED;
+  }
+  return AA_OK;
+}
+
+// The common checks plus the big-block geometry of the three AnchorAttention stages.
+int check_dims(const Dims& d, const char* who) {
+  if (int rc = check_common_dims(d, who)) return rc;
   if (d.block_size != 128) {
     set_error("%s: block_size %d is not supported (only 128)", who, d.block_size);
     return AA_EUNSUPPORTED;
@@ -49,14 +68,6 @@ int check_dims(const Dims& d, const char* who) {
   }
   if (d.n_ctx % (d.block_size * d.step) != 0) {
     set_error("%s: n_ctx %d is not a multiple of block_size*step = %d", who, d.n_ctx, d.block_size * d.step);
-    return AA_EUNSUPPORTED;
-  }
-  if (d.n_ctx > (1 << 20)) {
-    set_error("%s: n_ctx %d is larger than 1048576", who, d.n_ctx);
-    return AA_EUNSUPPORTED;
-  }
-  if ((int64_t)d.batch * d.n_q_heads * (d.n_ctx / 128) > 0x7fffffffLL) {
-    set_error("%s: problem too large for one launch", who);
     return AA_EUNSUPPORTED;
   }
   return AA_OK;
@@ -214,7 +225,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, float sm_scale, float theta_log2, int geometry, void* stream) {
+                     int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream) {
   const char* who = "aa_stage2_select";
   int rc;
   if (geometry != AA_GEOMETRY_AS_RUN && geometry != AA_GEOMETRY_INTENDED) {
@@ -234,7 +245,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
-  a.scale2 = (float)((double)sm_scale * 1.44269504);  // double product, then float32, as the definition does
+  a.scale2 = (float)(sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
   a.tile_lo = geometry == AA_GEOMETRY_AS_RUN ? 1 : step;
   a.tile_slack = geometry == AA_GEOMETRY_AS_RUN ? 2 : 1;
@@ -281,7 +292,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                       int block_size, int step, float sm_scale, float theta, int scale_mode, int geometry,
+                       int block_size, int step, double sm_scale, float theta_log2, int scale_mode, int geometry,
                        void* stream) {
   const char* who = "aa_anchor_attn_fwd";
   int rc;
@@ -302,16 +313,14 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   int32_t* coords = (int32_t*)(ws + w.coords);
   int32_t* counts = (int32_t*)(ws + w.counts);
   if ((rc = aa_stage1_anchor_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc, batch, n_q_heads,
-                                 n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, scale_mode, stream)))
+                                 n_kv_heads, n_ctx, head_dim, block_size, step, (float)sm_scale, scale_mode, stream)))
     return rc;
   if ((rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, stream))) return rc;
-  // theta -> log2 domain: a double product rounded to float32 (the definition multiplies a Python float)
-  const float theta_log2 = (float)((double)theta * 1.44269504);
   if ((rc = aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, mask, coords, counts, batch, n_q_heads, n_kv_heads, n_ctx,
                              head_dim, block_size, step, sm_scale, theta_log2, geometry, stream)))
     return rc;
   if ((rc = aa_stage3_sparse_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, coords, counts, M, L, acc, out,
-                                 o_sb, o_sh, o_sn, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale,
+                                 o_sb, o_sh, o_sn, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, (float)sm_scale,
                                  stream)))
     return rc;
   if (counts_out != nullptr) {
@@ -330,13 +339,7 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                         float sm_scale, void* stream) {
   const char* who = "aa_dense_causal_fwd";
   int rc;
-  if (n_ctx <= 0 || n_ctx % 128 != 0) {
-    set_error("%s: n_ctx %d must be a positive multiple of 128", who, n_ctx);
-    return AA_EUNSUPPORTED;
-  }
-  Dims d = {batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16};
-  d.n_ctx = 2048;  // only the generic checks; divisibility by the big block does not apply here
-  if ((rc = check_dims(d, who))) return rc;
+  if ((rc = check_common_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16}, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
   if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;

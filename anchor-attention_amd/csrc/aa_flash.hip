@@ -90,7 +90,9 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) { return (uint32_t)(
 // 64 lanes x 16 bytes, global -> LDS without passing through registers: lane L's bytes land at
 // lds_dst + 16*L (lds_dst is wave-uniform and travels in M0).  Completion is tracked by vmcnt.
 __device__ __forceinline__ void load16_to_lds(const char* base, const uint32_t byte_off, const uint32_t lds_dst) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_dst), "v"(byte_off), "s"(base) : "memory");
+  // the LDS base is bound to M0 by the constraint, so the compiler knows that M0 is written here; the nop covers the
+  // wait state an LDS-DMA instruction needs after a scalar write of M0 (the compiler does not look inside the asm)
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
 }
 
 // One K/V tile: wave w fills LDS rows 16*j + 4*w .. +3 (j = 0..3), i.e. thread t brings the chunk that belongs in

@@ -24,8 +24,9 @@ for _p in (ROOT, os.path.join(ROOT, "anchor-attention_amd")):
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/hbm_traffic_*.md); a counter
-# run cannot be made from inside this script, so the figure is carried here for the workload it was taken on
+# HBM bytes per launch measured with rocprofv3 FETCH_SIZE/WRITE_SIZE; a counter run cannot be made from inside
+# this script, so the figure is carried here for the workload it was taken on, with the file it was copied from
+TRAFFIC_SOURCE = "profiles/hbm_traffic_config2_llama8b_128k.md"
 MEASURED_TRAFFIC_BYTES = {
     "config2_llama8b_128k": {0: 4.53e9, 3: 4.36e9},  # dominant-kernel index -> bytes (stage 1, stage 3)
 }
@@ -235,6 +236,13 @@ def main():
         "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom) if (args.theta == 12.0 and args.qbar_mode == "shared") else None,
         "kernel_ms": st_ms[dom],
     }
+    roof["traffic_source"] = TRAFFIC_SOURCE if roof["traffic"] is not None else None
+    # stage 3 at this sparsity is bound by HBM (resume state in, output out), stage 2 and pooling likewise:
+    # algorithmic bytes per launch over the event-timed duration
+    b_pool = hq * n_ctx * D * 2 + hq * n_ctx * 4 + hq * (n_ctx // BS) * (D + 1) * 2
+    b2 = hkv * n_ctx * D * 2 + hq * (n_ctx // BS) * (D * 2 + 2 + 4) + 4 * sum_counts + 4 * hq * (n_ctx // S)
+    b3 = sum_counts * 2 * D * 2 + hq * n_ctx * D * 2 * 2 + 4 * sum_counts + hq * n_ctx * (D + 2) * 4
+    stage_gbs = {"pool": b_pool / st_ms[1] / 1e6, "stage2": b2 / st_ms[2] / 1e6, "stage3": b3 / st_ms[3] / 1e6}
     rec = {
         "metric": "anchor_attn_prefill_layer_effective_tflops",
         "value": (f1 + f2 + f3) / ms_per_step / 1e9,
@@ -254,7 +262,10 @@ def main():
         "computed_fraction_of_dense": (f1 + f3) / dense_flops,
         "stage_ms": {"stage1_anchor": st_ms[0], "pool": st_ms[1], "stage2_select": st_ms[2], "stage3_sparse": st_ms[3]},
         "stage_tflops": {"stage1": stage_tflops[0], "stage2": stage_tflops[2], "stage3": stage_tflops[3]},
+        "stage_hbm_gbs": stage_gbs,
+        "stage3_frac_of_hbm_peak": stage_gbs["stage3"] / PEAK_HBM_GBS,
         "flops": {"F1": f1, "F2": f2, "F3": f3, "dense_causal": dense_flops},
+        "algorithmic_bytes": {"pool": b_pool, "stage2": b2, "stage3": b3},
         "roofline": roof,
     }
     if not args.no_gemm_ref:

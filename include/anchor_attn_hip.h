@@ -96,15 +96,18 @@ int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, co
 /* Replaces anchor_attn_step_2 / get_q_mask / get_q_mask_triton (anchor_step_1_2_v2.py:199-210,
  * get_mask_test.py:7-159): key j in [block_size, bb*S - block_size) is selected for big block bb
  * iff for one of its pooled rows i  float(bf16(dot(qbar_i,k_j) * sm_scale*1.44269504)) + theta_log2
- * >= float(abar_i).  theta_log2 is theta * 1.44269504 (anchor_attn_v4.py:298).  geometry: AA_GEOMETRY_* (the
- * candidate range above is the as-run one).
+ * >= float(abar_i).  theta_log2 is float32(theta * 1.44269504), the product formed in double precision as the
+ * reference's entry does with Python floats (anchor_attn_v4.py:298) and handed to the kernel as a float32
+ * argument.  sm_scale is a double because the score scale is a compile-time constant in the reference's kernel:
+ * float32(double(sm_scale) * 1.44269504) (get_mask_test.py:86).  geometry: AA_GEOMETRY_* (the candidate range
+ * above is the as-run one).
  * mask_ws: scratch of aa_mask_words() uint32.  Outputs: coords (packed, see above) and
  * counts [B,Hq,N/S] int32.  Deterministic: no atomics, lists are ascending. */
 int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, float sm_scale, float theta_log2, int geometry, void* stream);
+                     int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream);
 
 /* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
  * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
@@ -124,14 +127,16 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
  * one stream.  workspace: aa_workspace_bytes() bytes of device scratch (contents undefined
  * afterwards).  counts_out (optional, may be NULL): [B,Hq,N/S] int32 copy of the per-big-block
  * selection counts, from which the caller forms the sparsity ratio (anchor_attn_v4.py:270-272).
- * theta is in natural-log units as in the reference's `difference` argument. */
+ * theta_log2 and the double sm_scale are those of aa_stage2_select (the caller forms theta * 1.44269504 in double
+ * precision, as anchor_attn_v4.py:298 does, so that the one-call and the staged paths see the same float32);
+ * stages 1 and 3 use float32(sm_scale), a run-time float32 argument of the reference's stage-3 kernel. */
 int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                        void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                       int block_size, int step, float sm_scale, float theta, int scale_mode, int geometry,
+                       int block_size, int step, double sm_scale, float theta_log2, int scale_mode, int geometry,
                        void* stream);
 
 /* ---- dense causal baseline on the same MFMA core --------------------------------------------

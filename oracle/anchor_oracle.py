@@ -22,8 +22,8 @@ multiplicity formula for double-counted keys.  The two query pre-scaling chains
 ``q3_scale_chain``: float32 products for stage 3, whose kernel takes it at run time) are pinned
 bit for bit against the Triton toolchain itself: tests/triton_promotion_probe.py compiles the two
 forms of the reference's expression as micro-kernels of its own, and its outputs on an MI355X are
-the fixture tests/golden/triton_scale_chain_probe.npz (Triton 3.6.0; the reference pins no Triton
-version).  ``stage1_scale_mode`` remains a switch.
+the fixture tests/golden/triton_scale_chain_probe.npz (made with Triton 3.6.0; the reference's
+requirements.txt pins 3.2.0, which is not installed here).  ``stage1_scale_mode`` remains a switch.
 
 Conventions: ``Q`` is ``[B, Hq, N, D]``, ``K``/``V`` are ``[B, Hkv, N, D]`` with ``Hkv | Hq``
 (query head ``h`` reads KV head ``h // (Hq // Hkv)``, the order ``repeat_kv`` produces);
@@ -173,9 +173,14 @@ def stage1_anchor(
 def pool_rows_f32_sequential(x: np.ndarray, block: int) -> np.ndarray:
     """Sum groups of ``block`` consecutive rows in float32, strictly in ascending row order.
 
-    The reference sums in float32 too (``tl.sum`` promotes bf16, get_mask_test.py:76-77,82-83)
-    without fixing an order; a sequential order is chosen here so that a kernel can reproduce it
-    bit for bit."""
+    The reference writes ``tl.sum(q, axis=1) / BLOCK_SZ`` on the loaded tile (get_mask_test.py:76-77,82-83)
+    and fixes neither the order nor, for the bf16 query tile, the accumulator type: that is a property
+    of the Triton release (releases up to 3.1 widened bf16 to float32 inside ``tl.sum``; 3.6.0 reduces
+    the bf16 tile in bf16; the reference pins 3.2.0, which is not available to check).  The anchors are
+    float32 and are summed in float32 by every release.  This oracle takes the float32 sum - the
+    closer of the two readings to the exact mean - in a sequential order, so that a kernel can
+    reproduce it bit for bit; what the other reading changes was measured (38 of 855 140 selected
+    indices and at most one bf16 step in the output at 128k tokens, tests/test_gpu_parity.py)."""
     n, c = x.shape
     xr = x.reshape(n // block, block, c)
     acc = np.zeros((n // block, c), np.float32)

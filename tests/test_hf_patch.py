@@ -32,6 +32,28 @@ def test_patch_model_validation_and_config():
     assert (m.config.block_size_M, m.config.step, m.config.theta) == (128, 16, 11)
     patch_model(m, "flash")
     assert m.config._attn_implementation == "sdpa"
+    # the reference's second name for the same forward and the same defaults (patch.py:41-45,142-144)
+    assert get_config_example("anchor_attn_lite") == get_config_example("anchor_attn")
+    patch_model(m, "anchor_attn_lite", {"theta": 13})
+    assert m.config._attn_implementation == "anchor_attn" and m.config.theta == 13
+    # dense attention on the package's own kernel
+    patch_model(m, "dense")
+    assert m.config._attn_implementation == "anchor_attn_dense"
+    assert set(get_config_example()) == {"default", "flash", "dense", "anchor_attn", "anchor_attn_lite"}
+
+
+def test_dense_pattern_on_cpu_is_plain_attention():
+    """Without a GPU the dense plug has only its framework branch; a model patched with it computes what the
+    unpatched model computes (prefill and cached decode)."""
+    from anchor_attn import patch_model
+    ref = _tiny()
+    m = _tiny()
+    m.load_state_dict(ref.state_dict())
+    patch_model(m, "dense")
+    x = torch.randint(0, 1000, (1, 200))
+    with torch.no_grad():
+        assert torch.allclose(ref(x).logits, m(x).logits, atol=1e-5)
+        assert torch.equal(ref.generate(x, max_new_tokens=3, do_sample=False), m.generate(x, max_new_tokens=3, do_sample=False))
 
 
 def test_short_prefill_and_decode_take_the_dense_branch():
@@ -71,7 +93,7 @@ def test_plug_dense_branch_matches_reference_math():
 # ------------------------------------------------------------------------------------ GPU
 @pytest.mark.gpu
 @pytest.mark.parametrize("n_tokens", [2 * 2048 + 300, 2 * 2048])
-def test_plug_sparse_branch_is_the_operator_plus_dense_tail(n_tokens):
+def test_plug_sparse_branch_is_the_operator_plus_dense_tail(n_tokens, monkeypatch):
     """The plug on HF-layout (transposed, non-contiguous) tensors = anchor_attn on contiguous copies for the
     rows the operator covers (bit for bit) + dense attention for the tail rows; pad == 0 included."""
     from anchor_attn.src.modules.llama import anchor_attention as aa
@@ -82,7 +104,12 @@ def test_plug_sparse_branch_is_the_operator_plus_dense_tail(n_tokens):
     # what LlamaAttention hands over: [B,H,N,D] views of [B,N,H,D] storage
     qh, kh, vh = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
     mod = types.SimpleNamespace(config=types.SimpleNamespace(block_size_M=128, step=16, theta=12.0))
+    aa.last_ratio = None
+    plain, _ = aa.anchor_attention_forward(mod, qh, kh, vh, None, scaling=128 ** -0.5)
+    assert aa.last_ratio is None  # by default the plug asks for no ratio, as the reference's caller does
+    monkeypatch.setattr(aa, "record_ratio", True)
     out, _ = aa.anchor_attention_forward(mod, qh, kh, vh, None, scaling=128 ** -0.5)
+    assert torch.equal(out, plain) and aa.last_ratio.is_cuda
     assert out.shape == (1, n_tokens, 4, 128) and out.is_contiguous()
     main = n_tokens - n_tokens % 2048
     want, ratio = anchor_attn(q[:, :, :main].contiguous(), k[:, :, :main].contiguous(), v[:, :, :main].contiguous())
@@ -114,7 +141,7 @@ def test_patched_model_equals_dense_model_when_the_window_covers_everything():
 
 
 @pytest.mark.gpu
-def test_patched_qwen2_model():
+def test_patched_qwen2_model(monkeypatch):
     """The same plug under Qwen2 (attention biases, its own config class): window-covers-everything equality with
     the dense model, and a real sparse prefill that stays finite and reports a ratio."""
     from transformers import Qwen2Config, Qwen2ForCausalLM
@@ -135,9 +162,98 @@ def test_patched_qwen2_model():
         b = m(x, logits_to_keep=32).logits.float()
     assert torch.isfinite(b).all() and (a - b).abs().max() < 0.08 * a.abs().max()
     patch_model(m, "anchor_attn", {"theta": 12})
+    import anchor_attn.src.modules.llama.anchor_attention as llama_plug
+    monkeypatch.setattr(llama_plug, "record_ratio", True)
     y = torch.randint(0, 1000, (1, 3 * 2048), device="cuda")
     with torch.no_grad():
         c = m(y, logits_to_keep=1).logits
-    import anchor_attn.src.modules.llama.anchor_attention as llama_plug
     assert torch.isfinite(c).all() and plug.anchor_attention_forward is llama_plug.anchor_attention_forward
     assert 0 < float(llama_plug.last_ratio) <= 1.0
+
+
+@pytest.mark.gpu
+def test_dense_plug_is_the_own_kernel_plus_tail():
+    """The dense plug on HF-layout tensors with a ragged length: rows below the last multiple of 128 come from
+    aa_dense_causal_fwd (bit for bit what dense_causal_attention returns), the tail from the framework; the whole
+    agrees with float64 library attention."""
+    from anchor_attn.src.modules.llama import anchor_attention as aa
+    from anchor_attn.src.ops.anchor_attn_v4 import dense_causal_attention
+    from anchor_attn.synthetic import make_qkv
+    n = 2048 + 128 + 37
+    q, k, v, _ = make_qkv(2048 + 256, 4, 2, n_stripes=16, seed=8)
+    q, k, v = (t[:, :, :n].cuda() for t in (q, k, v))
+    qh, kh, vh = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+    out, w = aa.dense_attention_forward(types.SimpleNamespace(config=None), qh, kh, vh, None, scaling=128 ** -0.5)
+    assert w is None and out.shape == (1, n, 4, 128) and out.is_contiguous()
+    main = n - n % 128
+    want = dense_causal_attention(q[:, :, :main].contiguous(), k[:, :, :main].contiguous(), v[:, :, :main].contiguous())
+    assert torch.equal(out.transpose(1, 2)[:, :, :main], want)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    err = (out.transpose(1, 2).double() - ref).abs()
+    assert err.max() < 2e-2 and err.mean() < 1e-3
+
+
+@pytest.mark.gpu
+def test_two_layer_llama8b_width_prefill_at_128k_all_patterns():
+    """BASELINE config 4 in small: the Llama-3.1-8B layer (hidden 4096, FFN 14336, 32/8 heads, vocab 128256, RoPE base
+    5e5) with random-init bf16 weights, two layers instead of 32, at the full 131072 tokens, through the three
+    patterns.  Every layer's attention goes through the plug exactly once; the sparse prefill causes no host
+    synchronisation inside the plug (the ratio stays on the device); logits are finite; the dense pattern (own
+    kernel) and the flash pattern (library attention) agree."""
+    from transformers import AttentionInterface, LlamaConfig, LlamaForCausalLM
+
+    from anchor_attn import patch_model
+    from anchor_attn.src.modules.llama import anchor_attention as plug
+    n_ctx, n_layers = 131072, 2
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=n_layers, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=n_ctx,
+                      rope_theta=5e5, tie_word_embeddings=False)
+    with torch.device("cuda"):
+        model = LlamaForCausalLM(cfg).to(torch.bfloat16).eval()
+    tokens = torch.randint(0, cfg.vocab_size, (1, n_ctx), device="cuda")
+    calls = {"anchor": 0, "dense": 0}
+    ratios = []
+    sparse_inner, dense_inner = plug.anchor_attention_forward, plug.dense_attention_forward
+
+    def sparse_counted(*a, **k):
+        calls["anchor"] += 1
+        torch.cuda.set_sync_debug_mode("error")  # any host<-device wait inside the plug raises
+        try:
+            r = sparse_inner(*a, **k)
+        finally:
+            torch.cuda.set_sync_debug_mode("default")
+        ratios.append(plug.last_ratio)
+        return r
+
+    def dense_counted(*a, **k):
+        calls["dense"] += 1
+        return dense_inner(*a, **k)
+
+    def prefill():
+        with torch.no_grad():
+            return model(tokens, use_cache=False, logits_to_keep=4).logits.float()
+
+    patch_model(model, "anchor_attn")
+    old_flag = plug.record_ratio
+    try:
+        plug.record_ratio = True
+        AttentionInterface.register(plug.ATTN_NAME, sparse_counted)
+        AttentionInterface.register(plug.DENSE_ATTN_NAME, dense_counted)
+        sparse = prefill()
+        assert calls == {"anchor": n_layers, "dense": 0}
+        assert all(r is not None and r.is_cuda and r.dim() == 0 for r in ratios)
+        assert all(0.0 < float(r) <= 1.0 for r in ratios)
+        patch_model(model, "dense")
+        dense = prefill()
+        assert calls == {"anchor": n_layers, "dense": n_layers}
+    finally:
+        plug.record_ratio = old_flag
+        AttentionInterface.register(plug.ATTN_NAME, sparse_inner)
+        AttentionInterface.register(plug.DENSE_ATTN_NAME, dense_inner)
+    patch_model(model, "flash")
+    flash = prefill()
+    assert torch.isfinite(sparse).all() and torch.isfinite(dense).all() and torch.isfinite(flash).all()
+    scale = flash.abs().max()
+    assert (dense - flash).abs().max() < 0.05 * scale and (dense - flash).abs().mean() < 0.01 * flash.abs().mean() + 1e-3
