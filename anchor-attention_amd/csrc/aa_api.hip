@@ -4,10 +4,16 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/anchor_attn_hip.h"
 #include "aa_common.h"
 #include "aa_kernels.h"
+
+// Device memory for aa_stage2_select_static(): the stage-2 bitmask and thresholds of callers that cannot
+// allocate.  Every GPU the library's code object is loaded on holds its own copy until the process ends.  In host
+// code this name only stands for the symbol; the memory's address on a device comes from hipGetSymbolAddress().
+static __device__ __align__(256) unsigned char scratch[AA_STATIC_SCRATCH_BYTES];
 
 namespace aa {
 
@@ -123,6 +129,32 @@ hipError_t run_flash(const FlashArgs& a, int mode, hipStream_t stream) {
 }
 
 size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+// Address of `scratch` on the current device, looked up once per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out, const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: cannot tell the current device (%s, device %d)", who, hipGetErrorString(e), dev);
+    return AA_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+      return AA_ELAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return AA_OK;
+}
 
 struct Workspace {
   size_t M, L, acc, qbar, abar, mask, coords, counts, total;
@@ -252,6 +284,27 @@ int aa_stage2_select(const void* qbar, const void* abar,
   if ((rc = check_launch(launch_select_thresholds(a, (hipStream_t)stream), who))) return rc;
   if ((rc = check_launch(launch_select_scores(a, (hipStream_t)stream), who))) return rc;
   return check_launch(launch_select_compact(a, (hipStream_t)stream), who);
+}
+
+int aa_stage2_select_static(const void* qbar, const void* abar,
+                            const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                            int32_t* coords, int32_t* counts,
+                            int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                            int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream) {
+  const char* who = "aa_stage2_select_static";
+  int rc;
+  if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  const int64_t need = aa_mask_words(batch, n_q_heads, n_ctx, block_size, step) * 4;
+  if (need > (int64_t)AA_STATIC_SCRATCH_BYTES) {
+    set_error("%s: this problem needs %lld bytes of stage-2 scratch, the static scratch holds %lld (batch*n_q_heads*n_ctx^2 too "
+              "large: use aa_stage2_select with a caller-provided buffer)", who, (long long)need, (long long)AA_STATIC_SCRATCH_BYTES);
+    return AA_EUNSUPPORTED;
+  }
+  void* ws = nullptr;
+  if ((rc = static_scratch(&ws, who))) return rc;
+  // from here on exactly aa_stage2_select: same checks, same kernels, the scratch pointer as an ordinary argument
+  return aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, static_cast<uint32_t*>(ws), coords, counts, batch, n_q_heads,
+                          n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, theta_log2, geometry, stream);
 }
 
 int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,

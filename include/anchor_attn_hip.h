@@ -109,6 +109,24 @@ int aa_stage2_select(const void* qbar, const void* abar,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
                      int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream);
 
+/* Same operation, same kernels and same results as aa_stage2_select, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc) and therefore cannot provide
+ * mask_ws: the bitmask and thresholds live in a static device array of AA_STATIC_SCRATCH_BYTES inside the library
+ * (one copy per GPU, held until the process ends).  This entry point has no counterpart in the reference, whose
+ * get_q_mask allocates its buffers with torch on every call (get_mask_test.py:138-145).
+ * It calls no hipMalloc/hipFree or other allocating routine.  Problems whose aa_mask_words()*4 exceeds
+ * AA_STATIC_SCRATCH_BYTES are refused with AA_EUNSUPPORTED (the Llama-3.1-8B layer at 131072 tokens, 32 query heads,
+ * needs 32.1 MiB and fits).  The first call on a device looks the array's address up (hipGetSymbolAddress): make
+ * that call outside any stream capture.  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls ordered on one stream do not.  Nothing has to be cleared between calls: every
+ * word stage 2 reads is written earlier in the same call. */
+#define AA_STATIC_SCRATCH_BYTES (40 * 1024 * 1024)
+int aa_stage2_select_static(const void* qbar, const void* abar,
+                            const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                            int32_t* coords, int32_t* counts,
+                            int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                            int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream);
+
 /* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
  * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
  * :246-268): resumes the online softmax from (M, L, acc_frag) over the K/V rows gathered at the
