@@ -22,7 +22,7 @@ ATTENTION_CONFIG_EXAMPLE = {
 }
 
 _SUPPORTED_MODELS = ("llama", "qwen2")
-SUPPORTED_BLOCK_SIZES = (128,)
+SUPPORTED_BLOCK_SIZES = (16, 32, 64, 128, 256)
 
 
 def get_config_example(pattern: str = None):

@@ -49,6 +49,7 @@ def _anchor_attn(Q, K, V, sm_scale=None, block_size=64, step=16, difference=100,
     here, as in the reference's private function, anchor_attn_v4.py:226-273)."""
     B, H, N, D = Q.shape
     assert N % block_size == 0
+    assert block_size in [16, 32, 64, 128, 256], "BLOCK_SIZE must be a power of 2 and ≥16"  # get_mask_test.py:133
     _check_inputs(Q, K, V)
     output = torch.empty_like(Q) if out is None else out
     assert output.shape == Q.shape and output.dtype == Q.dtype and output.stride(-1) == 1

@@ -64,8 +64,8 @@ int check_common_dims(const Dims& d, const char* who) {
 // The common checks plus the big-block geometry of the three AnchorAttention stages.
 int check_dims(const Dims& d, const char* who) {
   if (int rc = check_common_dims(d, who)) return rc;
-  if (d.block_size != 128) {
-    set_error("%s: block_size %d is not supported (only 128)", who, d.block_size);
+  if (d.block_size != 16 && d.block_size != 32 && d.block_size != 64 && d.block_size != 128 && d.block_size != 256) {
+    set_error("%s: block_size %d is not supported (16, 32, 64, 128 or 256)", who, d.block_size);
     return AA_EUNSUPPORTED;
   }
   if (d.step != 16 && d.step != 32) {
@@ -279,8 +279,16 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.big_block = block_size * step; a.block_size = block_size;
   a.scale2 = (float)(sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
-  a.tile_lo = geometry == AA_GEOMETRY_AS_RUN ? 1 : step;
-  a.tile_slack = geometry == AA_GEOMETRY_AS_RUN ? 2 : 1;
+  a.key_lo = geometry == AA_GEOMETRY_AS_RUN ? block_size : block_size * step;
+  a.key_slack = geometry == AA_GEOMETRY_AS_RUN ? block_size : 0;
+  // the score kernel numbers (query head of the KV group, big block) pairs with 16 bits and addresses the pooled
+  // queries with 32-bit byte offsets
+  if ((int64_t)(n_q_heads / n_kv_heads) * (n_ctx / (block_size * step)) >= 65536 ||
+      (int64_t)batch * n_q_heads * (n_ctx / block_size) * 256 > 0xffffffffLL) {
+    set_error("%s: too many (head, big block) pairs or pooled rows for one launch (heads per KV head %d, big blocks %d, pooled rows %lld)",
+              who, n_q_heads / n_kv_heads, n_ctx / (block_size * step), (long long)batch * n_q_heads * (n_ctx / block_size));
+    return AA_EUNSUPPORTED;
+  }
   if ((rc = check_launch(launch_select_thresholds(a, (hipStream_t)stream), who))) return rc;
   if ((rc = check_launch(launch_select_scores(a, (hipStream_t)stream), who))) return rc;
   return check_launch(launch_select_compact(a, (hipStream_t)stream), who);

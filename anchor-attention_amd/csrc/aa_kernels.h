@@ -36,8 +36,8 @@ struct SelectArgs {
   int batch, n_q_heads, n_kv_heads, n_ctx;
   int big_block, block_size;
   float scale2, theta_log2;
-  // candidate 128-key tiles of big block bb: tile_lo <= t <= step*bb - tile_slack (as run: 1 and 2; intended: step and 1)
-  int tile_lo, tile_slack;
+  // candidate keys of big block bb: key_lo <= j < bb*S - key_slack (as run: block_size and block_size; intended: S and 0)
+  int key_lo, key_slack;
 };
 hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream);
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream);

@@ -2,11 +2,11 @@
 //
 //  pool     qbar = bf16(mean of 128 raw query rows), abar = bf16(mean of 128 anchors); float32 sums in
 //           ascending row order so the result is reproducible bit for bit.
-//  scores   K-stationary: one work-group per (batch, KV head, 512 keys); each of its four waves keeps a
-//           128-key tile in registers as the MFMA B operand, and the pooled query rows of EVERY query
-//           head of the KV group and EVERY later big block stream past them (A operand, 32 pooled rows
-//           per MFMA, staged once per work-group in LDS).  Each K row is thus read once per KV head
-//           instead of once per (query head, big block).
+//  scores   K-stationary: one work-group per (batch, KV head, 256 keys); each of its four waves keeps 64
+//           keys in registers as the MFMA B operand, and the pooled query rows of EVERY query head of
+//           the KV group and EVERY later big block stream past them (A operand, 32 pooled rows per
+//           MFMA, staged once per work-group in LDS, 128 rows per barrier).  Each K row is thus read
+//           once per KV head instead of once per (query head, big block).
 //           In the 32x32 accumulator a lane holds one key column; OR-ing its registers over the pooled
 //           rows of a big block and a wave ballot give a 32-bit key mask per (q head, big block, key
 //           block) with no LDS and no atomics.
@@ -101,49 +101,77 @@ hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// STEP = pooled rows per big block (16 or 32); 32 / STEP (head, big block) items share one MFMA.
-// Work-group = 4 waves = 512 keys: wave w keeps key tile 4*T + w in registers (MFMA B operand) and all
-// four waves multiply the same stream of pooled-query groups, which is staged once per work-group in
-// LDS (double-buffered, one barrier per group) together with the groups' thresholds.
-constexpr int kARowStride = 136;  // bf16 per staged pooled-query row: 272 B, conflict-free for row-per-lane 16-byte reads
+// STEP = pooled rows per big block (16 or 32); an "item" is one (query head of the KV group, big block) pair, i.e.
+// STEP pooled rows that share one output mask word per 32 keys.
+//
+// Work-group = 4 waves = one super-tile of 256 keys: wave w keeps keys 64*w .. 64*w+63 of it in registers (MFMA B
+// operand, 64 VGPRs) for the whole kernel.  The items that can select those keys - every query head of the KV group
+// and every big block from bb_lo on - stream past them as the A operand.  The stream is cut into blocks of 128
+// pooled rows; a block travels global -> LDS by LDS-DMA loads (no registers, no LDS store instructions) one whole
+// block ahead of its use, so a block's loads have the time of 64 MFMAs per wave to land, and the work-group
+// synchronises once per block.  LDS rows are unpadded 256 bytes whose 16-byte chunks are XOR-swizzled with the row
+// number on the load side (a lane fetches the chunk that belongs in its slot), which makes the row-per-lane 16-byte
+// operand reads conflict-free.  The rows' thresholds ride along (4 bytes per row).
+//
+// Rows 32*w .. 32*w+31 of a block are brought in by wave w: they belong to 32/STEP whole items, so the item -> (head,
+// big block) arithmetic is wave-uniform.
+constexpr int kKB = 2;            // 32-key blocks a wave keeps in registers (64 keys, 64 VGPRs -> two work-groups per CU)
+constexpr int kBlockRows = 128;   // pooled rows staged per barrier
+constexpr int kSelRowBytes = 256; // one pooled row in LDS
 
-constexpr int kKB = 2;  // 32-key blocks a wave keeps in registers (2: 64 keys, 64 VGPRs -> two work-groups per CU)
+typedef __attribute__((address_space(3))) char sel_lds_char;
+__device__ __forceinline__ uint32_t sel_lds_addr(const void* p) { return (uint32_t)(uintptr_t)(sel_lds_char*)p; }
+// 64 lanes x 16 bytes (or x 4 bytes) global -> LDS; lane L's bytes land at lds_dst + 16*L (4*L).  lds_dst is wave-uniform
+// and travels in M0; the nop covers the wait state an LDS-DMA instruction needs after a scalar write of M0.
+__device__ __forceinline__ void sel_load16_to_lds(const char* base, const uint32_t byte_off, const uint32_t lds_dst) {
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void sel_load4_to_lds(const char* base, const uint32_t byte_off, const uint32_t lds_dst) {
+  asm volatile("s_nop 0\n\tglobal_load_lds_dword %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
+}
 
 template <int STEP>
 __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs p) {
-  constexpr int kItems = 32 / STEP;
-  constexpr int kWavesPerTile = 4 / kKB;      // waves that share one 128-key tile
+  constexpr int kItems = 32 / STEP;            // items per 32-row MFMA group (= items a wave brings in per block)
+  constexpr int kGroups = kBlockRows / 32;     // MFMA groups per block
+  constexpr int kWavesPerTile = 4 / kKB;       // waves that share one 128-key tile
   constexpr int kTilesPerWg = 4 / kWavesPerTile;
-  __shared__ __attribute__((aligned(16))) __bf16 a_lds[2][32 * kARowStride];
-  __shared__ __attribute__((aligned(16))) float thr_lds[2][32];
+  __shared__ __attribute__((aligned(16))) char a_lds[2][kBlockRows * kSelRowBytes];
+  __shared__ __attribute__((aligned(16))) float thr_lds[2][kBlockRows];
 
   // Work-groups are renumbered so that each XCD owns a contiguous range ordered (batch, KV head, super-tile): the
   // pooled queries a work-group streams are those of its KV head's query heads (1 MiB per KV head at 128k tokens),
   // which then stay in that XCD's L2 instead of every XCD cycling through all heads' pooled queries.
-  const int n_bb = p.n_ctx / p.big_block;
+  const int S = p.big_block;
+  const int n_bb = p.n_ctx / S;
   const int n_t = p.n_ctx / 128;
   const int n_super = n_t / kTilesPerWg;
   uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, n_super, 1);
   const int T = vid % n_super;  // key super-tile (kTilesPerWg * 128 keys); ascending = heaviest first
   vid /= n_super;
   const int kvh = vid % p.n_kv_heads, b = vid / p.n_kv_heads;
-  const int n_pr = n_t;  // pooled rows per head (block_size == 128)
+  const int n_pr = p.n_ctx / p.block_size;  // pooled rows per head
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, c32 = lane & 31;
 
-  // key tile t is a candidate for big block bb iff tile_lo <= t <= STEP*bb - tile_slack,
-  // i.e. t >= tile_lo and bb >= (t + tile_slack + STEP - 1) / STEP
-  const int tw = kTilesPerWg * T + wave / kWavesPerTile;          // this wave's 128-key tile
-  const int kb0 = kKB * (wave % kWavesPerTile);                   // its first 32-key block inside the tile
-  const int bb_min_w = tw < p.tile_lo ? n_bb : (tw + p.tile_slack + STEP - 1) / STEP;
-  if (kTilesPerWg * T + kTilesPerWg - 1 < p.tile_lo) return;      // no tile of the work-group is ever a candidate
-  const int t_first = max(p.tile_lo, kTilesPerWg * T);            // first candidate tile of the work-group
-  const int bb_lo = (t_first + p.tile_slack + STEP - 1) / STEP;   // smallest big block any wave needs
+  // Key tile t (keys 128t .. 128t+127) holds candidates of big block bb iff it reaches past key_lo and starts below
+  // bb*S - key_slack, i.e. bb >= (128t + key_slack) / S + 1.
+  auto tile_bb_min = [&](const int t) { return 128 * t + 128 > p.key_lo ? (128 * t + p.key_slack) / S + 1 : n_bb; };
+  const int tw = kTilesPerWg * T + wave / kWavesPerTile;  // this wave's 128-key tile
+  const int kb0 = kKB * (wave % kWavesPerTile);           // its first 32-key block inside the tile
+  const int bb_min_w = tile_bb_min(tw);
+  int bb_lo = n_bb;                                       // smallest big block any wave of the work-group needs
+#pragma unroll
+  for (int i = 0; i < kTilesPerWg; ++i) bb_lo = min(bb_lo, tile_bb_min(kTilesPerWg * T + i));
   if (bb_lo >= n_bb) return;
   const int group = p.n_q_heads / p.n_kv_heads;
   const int n_items = group * (n_bb - bb_lo);
-  const int n_groups = (n_items + kItems - 1) / kItems;
+  const int n_blocks = (n_items * STEP + kBlockRows - 1) / kBlockRows;
+  // item -> (head in group, big block): item / group = floor(2*item * ceil(2^31 / group) / 2^32), exact for item < 2^16
+  // and group < 2^15 (the host checks both)
+  const uint32_t magic = (0x80000000u + (uint32_t)group - 1u) / (uint32_t)group;
+  auto item_bb_off = [&](const int item) { return (int)__umulhi(2u * (uint32_t)item, magic); };
 
   const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
   bf16x8 kreg[kKB][8];
@@ -154,98 +182,108 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
     for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
   }
 
-  // staging: thread t carries 32 bytes (chunks 2*(t&7), 2*(t&7)+1) of pooled row t>>3 of the group; row r of a
-  // group is pooled row (r % STEP) of item grp*kItems + r/STEP; threads 0..31 also carry the row's threshold
-  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-  u32x4 st0, st1;
-  float st_thr = 0.f;
-  auto stage_load = [&](const int grp) {
-    const int r = tid >> 3;
-    const int item = min(grp * kItems + r / STEP, n_items - 1);
-    const int64_t prow = ((int64_t)b * p.n_q_heads + kvh * group + item % group) * n_pr + (bb_lo + item / group) * STEP + r % STEP;
-    const __bf16* src = p.qbar + prow * 128 + 16 * (tid & 7);
-    st0 = *reinterpret_cast<const u32x4*>(src);
-    st1 = *reinterpret_cast<const u32x4*>(src + 8);
-    if (tid < 32) {
-      const int item2 = min(grp * kItems + tid / STEP, n_items - 1);
-      st_thr = p.thr[((int64_t)b * p.n_q_heads + kvh * group + item2 % group) * n_pr + (bb_lo + item2 / group) * STEP + tid % STEP];
-    }
-  };
-  auto stage_store = [&](const int buf) {
-    __bf16* dst = &a_lds[buf][(tid >> 3) * kARowStride + 16 * (tid & 7)];
-    *reinterpret_cast<u32x4*>(dst) = st0;
-    *reinterpret_cast<u32x4*>(dst + 8) = st1;
-    if (tid < 32) thr_lds[buf][tid] = st_thr;
-  };
-
-  stage_load(0);
-  stage_store(0);
-  __syncthreads();
-
-  for (int grp = 0; grp < n_groups; ++grp) {
-    const int buf = grp & 1;
-    if (grp + 1 < n_groups) stage_load(grp + 1);
-
-    // does this wave's key tile belong to the candidate range of either item of the group?
-    bool item_ok[kItems];
-    bool any_ok = false;
+  // ---- staging -------------------------------------------------------------------------------
+  // Load j (0..7) of wave w fills block rows 32w + 4j + (lane >> 4); lane brings chunk (lane & 15) ^ (row & 15).
+  const char* qbar_base = reinterpret_cast<const char*>(p.qbar);
+  const char* thr_base = reinterpret_cast<const char*>(p.thr);
+  const int64_t head0 = ((int64_t)b * p.n_q_heads + kvh * group) * n_pr;  // first pooled row of the group's first head
+  const uint32_t a_lds0 = sel_lds_addr(a_lds[0]) + wave * 32 * kSelRowBytes;
+  const uint32_t thr_lds0 = sel_lds_addr(thr_lds[0]);
+  auto stage_block = [&](const int blk, const int buf) {
+    // pooled-row number (within the whole qbar array) of the first row of each item this wave brings in
+    uint32_t item_row0[kItems];
 #pragma unroll
     for (int it = 0; it < kItems; ++it) {
-      const int item = grp * kItems + it;
-      item_ok[it] = item < n_items && (bb_lo + item / group) >= bb_min_w;
-      any_ok |= item_ok[it];
+      const int item = min(blk * (kGroups * kItems) + wave * kItems + it, n_items - 1);  // past the end: repeat the last item
+      const int q = item_bb_off(item);
+      item_row0[it] = (uint32_t)(head0 + (int64_t)(item - q * group) * n_pr + (int64_t)(bb_lo + q) * STEP);
     }
-    if (any_ok) {
-      bf16x8 a[8];
-      const __bf16* arow = &a_lds[buf][c32 * kARowStride + 8 * half];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) a[ks] = *reinterpret_cast<const bf16x8*>(arow + 16 * ks);
+    for (int j = 0; j < 8; ++j) {
+      const int r = 4 * j + (lane >> 4);  // row inside the wave's 32
+      const uint32_t prow = item_row0[r / STEP] + (uint32_t)(r % STEP);
+      const uint32_t chunk = (uint32_t)((lane & 15) ^ (r & 15));
+      sel_load16_to_lds(qbar_base, prow * (uint32_t)kSelRowBytes + chunk * 16u, a_lds0 + buf * (kBlockRows * kSelRowBytes) + 4 * j * kSelRowBytes);
+    }
+    if (wave < 2) {  // thresholds of block rows 64*wave + lane
+      const int r = 64 * wave + lane;
+      const int item = min(blk * (kGroups * kItems) + r / STEP, n_items - 1);
+      const int q = item_bb_off(item);
+      const uint32_t prow = (uint32_t)(head0 + (int64_t)(item - q * group) * n_pr + (int64_t)(bb_lo + q) * STEP) + (uint32_t)(r % STEP);
+      sel_load4_to_lds(thr_base, prow * 4u, thr_lds0 + buf * (kBlockRows * 4) + wave * 256);
+    }
+  };
+
+  stage_block(0, 0);
+
+  // A operand of MFMA step ks: row c32 of the group, chunk 2*ks + half, swizzled with the row's low four bits
+  uint32_t a_rd[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) a_rd[ks] = sel_lds_addr(a_lds[0]) + c32 * kSelRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8_t;
+  typedef __attribute__((address_space(3))) floatx4 lds_floatx4_t;
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+  constexpr int kBlockItems = kGroups * kItems;  // items per block (8 or 4): lane i < kBlockItems stores item i's words
+  for (int blk = 0; blk < n_blocks; ++blk) {
+    const int buf = blk & 1;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of block blk has landed
+    __syncthreads();                                   // ... and everyone's; everyone is done with the other buffer
+    if (blk + 1 < n_blocks) stage_block(blk + 1, buf ^ 1);
+    const uint32_t a_off = buf * (kBlockRows * kSelRowBytes);
+    // The four groups are straight-line code (no branch between them), so that the operand reads of one group can
+    // overlap the products of the previous one.  Every item is computed, also the few that cannot select this wave's
+    // keys (a big block below the tile's first one, the padding past the last item): those are simply not stored.
+    // The mask words of item i (wave-uniform ballot results) are dropped into lane i of w_lo / w_hi.
+    uint32_t w_lo = 0u, w_hi = 0u;
+#pragma unroll
+    for (int gi = 0; gi < kGroups; ++gi) {
+      bf16x8 a[8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) a[ks] = *(const lds_bf16x8_t*)(uintptr_t)(a_rd[ks] + a_off + gi * 32 * kSelRowBytes);
       // raw-score thresholds of the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
       float thr[16];
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        const floatx4 w = *reinterpret_cast<const floatx4*>(&thr_lds[buf][8 * rq + 4 * half]);
+        const floatx4 w = *(const lds_floatx4_t*)(uintptr_t)(thr_lds0 + buf * (kBlockRows * 4) + (32 * gi + 8 * rq + 4 * half) * 4);
         thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
         thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
       }
-      uint32_t words[kItems][kKB];
+      floatx16 c[kKB];
+      const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kb = 0; kb < kKB; ++kb) c[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kreg[kb][0], zero, 0, 0, 0);
+#pragma unroll
+      for (int ks = 1; ks < 8; ++ks)
+#pragma unroll
+        for (int kb = 0; kb < kKB; ++kb) c[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c[kb], 0, 0, 0);
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb) {
-        const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        floatx16 c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kreg[kb][0], zero, 0, 0, 0);
-#pragma unroll
-        for (int ks = 1; ks < 8; ++ks) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c, 0, 0, 0);
         bool hit[kItems];
 #pragma unroll
         for (int it = 0; it < kItems; ++it) hit[it] = false;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) hit[(8 * (r >> 2)) / STEP] |= (c[r] >= thr[r]);  // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
+        for (int r = 0; r < 16; ++r) hit[(8 * (r >> 2)) / STEP] |= (c[kb][r] >= thr[r]);  // rows 0..15 -> item 0, 16..31 -> item 1 (STEP 16)
 #pragma unroll
         for (int it = 0; it < kItems; ++it) {
           const uint64_t m = __ballot(hit[it]);
-          words[it][kb] = (uint32_t)m | (uint32_t)(m >> 32);  // both halves of the wave hold the same keys
-        }
-      }
-      if (lane == 0) {
-#pragma unroll
-        for (int it = 0; it < kItems; ++it) {
-          if (item_ok[it]) {
-            const int item = grp * kItems + it;
-            const int hq = kvh * group + item % group;
-            const int bb = bb_lo + item / group;
-            uint32_t* dst = p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + tw) * 4 + kb0;
-            if (kKB == 4) {
-              *reinterpret_cast<u32x4*>(dst) = u32x4{words[it][0], words[it][1], words[it][kKB - 2], words[it][kKB - 1]};
-            } else {
-              *reinterpret_cast<u32x2*>(dst) = u32x2{words[it][0], words[it][1]};
-            }
-          }
+          const uint32_t word = (uint32_t)m | (uint32_t)(m >> 32);  // both halves of the wave hold the same keys
+          if (kb == 0) w_lo = lane == gi * kItems + it ? word : w_lo;
+          else w_hi = lane == gi * kItems + it ? word : w_hi;
         }
       }
     }
-    if (grp + 1 < n_groups) stage_store(buf ^ 1);
-    __syncthreads();
+    // lane i stores the two words (this wave's 64 keys) of item blk * kBlockItems + i
+    if (lane < kBlockItems) {
+      const int item = blk * kBlockItems + lane;
+      const int q = item_bb_off(min(item, n_items - 1));
+      const int bb = bb_lo + q;
+      const int hq = kvh * group + (min(item, n_items - 1) - q * group);
+      if (item < n_items && bb >= bb_min_w) {
+        uint32_t* dst = p.mask + ((((int64_t)b * p.n_q_heads + hq) * n_bb + bb) * n_t + tw) * 4 + kb0;
+        *reinterpret_cast<u32x2*>(dst) = u32x2{w_lo, w_hi};
+      }
+    }
   }
 }
 
@@ -258,22 +296,27 @@ hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// One wave per (batch, query head, big block): the candidate keys [key_lo, bb*S - key_slack) of the big block's mask row
+// become an ascending index list (popcount per 32-key word, wave prefix sum, each lane writes its word's set bits).
 __global__ void __launch_bounds__(64) select_compact_kernel(const SelectArgs p) {
   const int bb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x;
   const int n_bb = p.n_ctx / p.big_block;
   const int n_t = p.n_ctx / 128;
-  const int step = p.big_block / p.block_size;
   const int64_t bh = (int64_t)b * p.n_q_heads + h;
-  const int t_lo = p.tile_lo, t_hi = step * bb - p.tile_slack;  // candidate key tiles, inclusive
+  const int key_lo = p.key_lo, key_hi = bb * p.big_block - p.key_slack;  // candidate keys [key_lo, key_hi)
   int base = 0;
-  if (t_hi >= t_lo) {
-    const int n_words = 4 * (t_hi - t_lo + 1);
-    const uint32_t* mw = p.mask + ((bh * n_bb + bb) * n_t + t_lo) * 4;
+  if (key_hi > key_lo) {
+    const int w_lo = key_lo / 32, w_hi = (key_hi + 31) / 32;  // mask words [w_lo, w_hi) of the row
+    const uint32_t* mw = p.mask + (bh * n_bb + bb) * n_t * 4;
     int32_t* out = p.coords + bh * p.coords_per_head + coords_tri(bb, p.big_block, p.block_size);
-    for (int w0 = 0; w0 < n_words; w0 += 64) {
+    for (int w0 = w_lo; w0 < w_hi; w0 += 64) {
       const int wi = w0 + lane;
-      uint32_t word = wi < n_words ? mw[wi] : 0u;
+      uint32_t word = wi < w_hi ? mw[wi] : 0u;
+      // the first and the last word may reach outside the candidate range (block sizes below 32 keys)
+      const int k0 = wi * 32;
+      if (k0 < key_lo) word &= key_lo - k0 >= 32 ? 0u : ~0u << (key_lo - k0);
+      if (k0 + 32 > key_hi) word &= key_hi <= k0 ? 0u : ~0u >> (k0 + 32 - key_hi);
       const int pc = __popc(word);
       int incl = pc;
 #pragma unroll
@@ -282,9 +325,8 @@ __global__ void __launch_bounds__(64) select_compact_kernel(const SelectArgs p) 
         if (lane >= d) incl += up;
       }
       int pos = base + incl - pc;
-      const int key_base = t_lo * 128 + wi * 32;
       while (word) {
-        out[pos++] = key_base + (__ffs(word) - 1);
+        out[pos++] = k0 + (__ffs(word) - 1);
         word &= word - 1;
       }
       base += __shfl(incl, 63, 64);

@@ -44,7 +44,7 @@ def llama_small(mods):
     return (q.cuda(), k.cuda(), v.cuda()), (Q, K, V), res
 
 
-def _packed_lists(hip, coords, counts, N, step=STEP):
+def _packed_lists(hip, coords, counts, N, step=STEP, bs=BS):
     coords = coords.cpu().numpy()
     counts = counts.cpu().numpy().reshape(coords.shape[0], coords.shape[1], -1)
     lib = hip.lib()
@@ -54,16 +54,16 @@ def _packed_lists(hip, coords, counts, N, step=STEP):
         for h in range(coords.shape[1]):
             ph = []
             for bb in range(counts.shape[2]):
-                off = lib.aa_coords_offset(bb, BS, step)
+                off = lib.aa_coords_offset(bb, bs, step)
                 ph.append(coords[b, h, off:off + counts[b, h, bb]].copy())
             pb.append(ph)
         out.append(pb)
     return out, counts
 
 
-def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP):
+def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP, bs=BS):
     """Sets equal except excused keys (flip distance < BAND); returns number of excused keys."""
-    S = BS * step
+    S = bs * step
     B, Hq = got_counts.shape[:2]
     group = Hq // K.shape[1]
     excused = 0
@@ -74,13 +74,13 @@ def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused,
                 g, w = got[b][h][bb], want[b][h][bb]
                 assert np.all(np.diff(g) > 0), "index list must be strictly ascending"
                 if g.size:
-                    assert g[0] >= BS and g[-1] < bb * S - BS
+                    assert g[0] >= bs and g[-1] < bb * S - bs
                 sym = np.setxor1d(g, w)
                 if sym.size == 0:
                     continue
                 if qbar is None:
-                    qbar = ao.pooled_queries(Q[b, h], BS)
-                    abar, mean = ao.pooled_anchors(M[b, h], BS)
+                    qbar = ao.pooled_queries(Q[b, h], bs)
+                    abar, mean = ao.pooled_anchors(M[b, h], bs)
                 rows = slice(bb * step, (bb + 1) * step)
                 for j in sym:
                     d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta)
@@ -176,21 +176,22 @@ def test_stage3_matches_oracle_given_same_state(mods, llama_small):
 
 
 # ------------------------------------------------------------------------------------ whole operator
-def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP):
+def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP, bs=BS):
     hip, v4, st, ao = mods
     Q, K, V = _np(q, k, v)
-    res = ao.anchor_attn_reference(Q, K, V, step=step, difference=theta)
+    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
-    out, ratio = v4.anchor_attn(qd, kd, vd, step=step, difference=theta)
+    out, ratio = v4.anchor_attn(qd, kd, vd, block_size=bs, step=step, difference=theta)
     B, H, N, _ = q.shape
     # stage outputs for index parity come from the staged entry points on the same inputs
-    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, step, B, H, N, D, SM)
-    coords, counts = st.select_stripes_packed(qd, kd, M, BS, step, theta * LOG2E, B, H, N, D, SM)
-    got, got_counts = _packed_lists(hip, coords, counts, N, step)
-    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step)
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, bs, step, B, H, N, D, SM)
+    np.testing.assert_allclose(M.cpu().numpy(), res.M, atol=3e-4)
+    coords, counts = st.select_stripes_packed(qd, kd, M, bs, step, theta * LOG2E, B, H, N, D, SM)
+    got, got_counts = _packed_lists(hip, coords, counts, N, step, bs)
+    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step, bs)
     err = np.abs(out.float().cpu().numpy() - res.out)
     assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
-    want_ratio = got_counts.sum() / ((B * H * N * N / (BS * step)) // 2)
+    want_ratio = got_counts.sum() / ((B * H * N * N / (bs * step)) // 2)
     assert abs(float(ratio) - want_ratio) < 1e-6
     return res, out
 
@@ -264,6 +265,23 @@ def test_assorted_shapes_and_thresholds(mods, n_bb, hq, hkv, step, theta, seed, 
     """Head groupings 1:1 to 8:1, both step sizes, thresholds from 8 to 16, three RoPE bases, both stripe laws."""
     q, k, v, _ = _case(n_bb * BS * step, hq, hkv, 40 * n_bb, seed=seed, rope_base=base, stripe_dist=dist)
     _end_to_end(mods, q, k, v, theta, max_excused=8, step=step)
+
+
+@pytest.mark.parametrize("bs,step,n_bb,hq,hkv,theta,seed", [
+    (64, 16, 5, 4, 2, 12.0, 201),    # the private _anchor_attn default of the reference (anchor_attn_v4.py:228)
+    (64, 32, 3, 2, 1, 13.0, 202),
+    (32, 16, 9, 2, 2, 12.0, 203),    # S = 512
+    (16, 16, 17, 3, 1, 11.0, 204),   # S = 256: two query blocks per big block, candidate range ends inside a 32-key word
+    (16, 32, 6, 2, 1, 12.0, 205),
+    (256, 16, 3, 4, 2, 12.0, 206),   # S = 4096, two work-groups of stage 1 per pooled row
+    (256, 32, 2, 1, 1, 14.0, 207),   # S = 8192
+])
+def test_other_block_sizes(mods, bs, step, n_bb, hq, hkv, theta, seed):
+    """Every block size the reference's assertion admits (get_mask_test.py:133): pooling over block_size rows,
+    candidates [block_size, bb*S - block_size), big block S = block_size * step."""
+    q, k, v, _ = _case(n_bb * bs * step, hq, hkv, max(8, n_bb * bs * step // 100), seed=seed)
+    res, _ = _end_to_end(mods, q, k, v, theta, max_excused=8, step=step, bs=bs)
+    assert res.counts.sum() > 0 and res.counts[:, :, 0].sum() == 0
 
 
 def test_theta_minus_inf_two_big_blocks_equals_library_attention(mods):
@@ -378,8 +396,8 @@ def test_entry_assertions_and_error_codes(mods):
         v4.anchor_attn(q[:, :, :1024], q[:, :, :1024], q[:, :, :1024])
     with pytest.raises(AssertionError):
         v4.anchor_attn(q.float(), q.float(), q.float())
-    with pytest.raises(hip.AnchorAttnHipError):
-        v4.anchor_attn(q, q, q, block_size=64, step=32)  # block_size 64 is not built
+    with pytest.raises(AssertionError):
+        v4.anchor_attn(q[:, :, :1536], q[:, :, :1536], q[:, :, :1536], block_size=48, step=16)  # not one of 16 ... 256
     lib = hip.lib()
     rc = lib.aa_dense_causal_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 2, 2048, 128, 0.1, None)
     assert rc == 1 and b"NULL" in lib.aa_last_error()
