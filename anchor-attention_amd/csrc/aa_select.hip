@@ -115,9 +115,17 @@ hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
 //
 // Rows 32*w .. 32*w+31 of a block are brought in by wave w: they belong to 32/STEP whole items, so the item -> (head,
 // big block) arithmetic is wave-uniform.
-constexpr int kKB = 2;            // 32-key blocks a wave keeps in registers (64 keys, 64 VGPRs -> two work-groups per CU)
-constexpr int kBlockRows = 128;   // pooled rows staged per barrier
+constexpr int kKB = 2;            // 32-key blocks a wave keeps in registers (64 keys, 64 VGPRs)
 constexpr int kSelRowBytes = 256; // one pooled row in LDS
+#ifndef AA_SEL_WAVES
+#define AA_SEL_WAVES 4            // waves per work-group (two waves share a 128-key tile)
+#endif
+#ifndef AA_SEL_ROWS
+#define AA_SEL_ROWS 128           // pooled rows staged per barrier
+#endif
+#ifndef AA_SEL_WGS
+#define AA_SEL_WGS 2              // work-groups per CU the kernel is compiled for
+#endif
 
 typedef __attribute__((address_space(3))) char sel_lds_char;
 __device__ __forceinline__ uint32_t sel_lds_addr(const void* p) { return (uint32_t)(uintptr_t)(sel_lds_char*)p; }
@@ -130,14 +138,18 @@ __device__ __forceinline__ void sel_load4_to_lds(const char* base, const uint32_
   asm volatile("s_nop 0\n\tglobal_load_lds_dword %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
 }
 
-template <int STEP>
-__global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs p) {
-  constexpr int kItems = 32 / STEP;            // items per 32-row MFMA group (= items a wave brings in per block)
-  constexpr int kGroups = kBlockRows / 32;     // MFMA groups per block
-  constexpr int kWavesPerTile = 4 / kKB;       // waves that share one 128-key tile
-  constexpr int kTilesPerWg = 4 / kWavesPerTile;
-  __shared__ __attribute__((aligned(16))) char a_lds[2][kBlockRows * kSelRowBytes];
-  __shared__ __attribute__((aligned(16))) float thr_lds[2][kBlockRows];
+template <int STEP, int WAVES, int ROWS>
+__global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(const SelectArgs p) {
+  constexpr int kItems = 32 / STEP;              // items per 32-row MFMA group
+  constexpr int kGroups = ROWS / 32;             // MFMA groups per block
+  constexpr int kBlockItems = ROWS / STEP;       // items per block
+  constexpr int kRowsPerWave = ROWS / WAVES;     // rows of a block a wave brings in
+  constexpr int kItemsPerWave = kRowsPerWave / STEP;
+  constexpr int kTilesPerWg = WAVES / 2;         // two waves share one 128-key tile
+  static_assert(kRowsPerWave % STEP == 0 && kItemsPerWave >= 1 && kRowsPerWave % 4 == 0, "a wave stages whole items");
+  static_assert(ROWS % 64 == 0 && ROWS / 64 <= WAVES, "thresholds are staged 64 per wave");
+  __shared__ __attribute__((aligned(16))) char a_lds[2][ROWS * kSelRowBytes];
+  __shared__ __attribute__((aligned(16))) float thr_lds[2][ROWS];
 
   // Work-groups are renumbered so that each XCD owns a contiguous range ordered (batch, KV head, super-tile): the
   // pooled queries a work-group streams are those of its KV head's query heads (1 MiB per KV head at 128k tokens),
@@ -158,16 +170,16 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   // Key tile t (keys 128t .. 128t+127) holds candidates of big block bb iff it reaches past key_lo and starts below
   // bb*S - key_slack, i.e. bb >= (128t + key_slack) / S + 1.
   auto tile_bb_min = [&](const int t) { return 128 * t + 128 > p.key_lo ? (128 * t + p.key_slack) / S + 1 : n_bb; };
-  const int tw = kTilesPerWg * T + wave / kWavesPerTile;  // this wave's 128-key tile
-  const int kb0 = kKB * (wave % kWavesPerTile);           // its first 32-key block inside the tile
+  const int tw = kTilesPerWg * T + wave / 2;  // this wave's 128-key tile
+  const int kb0 = kKB * (wave % 2);           // its first 32-key block inside the tile
   const int bb_min_w = tile_bb_min(tw);
-  int bb_lo = n_bb;                                       // smallest big block any wave of the work-group needs
+  int bb_lo = n_bb;                           // smallest big block any wave of the work-group needs
 #pragma unroll
   for (int i = 0; i < kTilesPerWg; ++i) bb_lo = min(bb_lo, tile_bb_min(kTilesPerWg * T + i));
   if (bb_lo >= n_bb) return;
   const int group = p.n_q_heads / p.n_kv_heads;
   const int n_items = group * (n_bb - bb_lo);
-  const int n_blocks = (n_items * STEP + kBlockRows - 1) / kBlockRows;
+  const int n_blocks = (n_items * STEP + ROWS - 1) / ROWS;
   // item -> (head in group, big block): item / group = floor(2*item * ceil(2^31 / group) / 2^32), exact for item < 2^16
   // and group < 2^15 (the host checks both)
   const uint32_t magic = (0x80000000u + (uint32_t)group - 1u) / (uint32_t)group;
@@ -183,34 +195,33 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   }
 
   // ---- staging -------------------------------------------------------------------------------
-  // Load j (0..7) of wave w fills block rows 32w + 4j + (lane >> 4); lane brings chunk (lane & 15) ^ (row & 15).
+  // Wave w brings in block rows w*kRowsPerWave ..: its load j fills rows 4j + (lane >> 4) of those; a lane brings
+  // chunk (lane & 15) ^ (row & 15).  The rows of one wave are whole items, so the item arithmetic is wave-uniform.
   const char* qbar_base = reinterpret_cast<const char*>(p.qbar);
   const char* thr_base = reinterpret_cast<const char*>(p.thr);
   const int64_t head0 = ((int64_t)b * p.n_q_heads + kvh * group) * n_pr;  // first pooled row of the group's first head
-  const uint32_t a_lds0 = sel_lds_addr(a_lds[0]) + wave * 32 * kSelRowBytes;
+  const uint32_t a_lds0 = sel_lds_addr(a_lds[0]) + wave * kRowsPerWave * kSelRowBytes;
   const uint32_t thr_lds0 = sel_lds_addr(thr_lds[0]);
+  auto item_first_row = [&](const int item_unclamped) {  // pooled-row number, within the whole qbar array, of an item's first row
+    const int item = min(item_unclamped, n_items - 1);   // past the end: repeat the last item
+    const int q = item_bb_off(item);
+    return (uint32_t)(head0 + (int64_t)(item - q * group) * n_pr + (int64_t)(bb_lo + q) * STEP);
+  };
   auto stage_block = [&](const int blk, const int buf) {
-    // pooled-row number (within the whole qbar array) of the first row of each item this wave brings in
-    uint32_t item_row0[kItems];
+    uint32_t item_row0[kItemsPerWave];
 #pragma unroll
-    for (int it = 0; it < kItems; ++it) {
-      const int item = min(blk * (kGroups * kItems) + wave * kItems + it, n_items - 1);  // past the end: repeat the last item
-      const int q = item_bb_off(item);
-      item_row0[it] = (uint32_t)(head0 + (int64_t)(item - q * group) * n_pr + (int64_t)(bb_lo + q) * STEP);
-    }
+    for (int it = 0; it < kItemsPerWave; ++it) item_row0[it] = item_first_row(blk * kBlockItems + wave * kItemsPerWave + it);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int r = 4 * j + (lane >> 4);  // row inside the wave's 32
+    for (int j = 0; j < kRowsPerWave / 4; ++j) {
+      const int r = 4 * j + (lane >> 4);  // row inside the wave's share
       const uint32_t prow = item_row0[r / STEP] + (uint32_t)(r % STEP);
       const uint32_t chunk = (uint32_t)((lane & 15) ^ (r & 15));
-      sel_load16_to_lds(qbar_base, prow * (uint32_t)kSelRowBytes + chunk * 16u, a_lds0 + buf * (kBlockRows * kSelRowBytes) + 4 * j * kSelRowBytes);
+      sel_load16_to_lds(qbar_base, prow * (uint32_t)kSelRowBytes + chunk * 16u, a_lds0 + buf * (ROWS * kSelRowBytes) + 4 * j * kSelRowBytes);
     }
-    if (wave < 2) {  // thresholds of block rows 64*wave + lane
+    if (wave < ROWS / 64) {  // thresholds of block rows 64*wave + lane
       const int r = 64 * wave + lane;
-      const int item = min(blk * (kGroups * kItems) + r / STEP, n_items - 1);
-      const int q = item_bb_off(item);
-      const uint32_t prow = (uint32_t)(head0 + (int64_t)(item - q * group) * n_pr + (int64_t)(bb_lo + q) * STEP) + (uint32_t)(r % STEP);
-      sel_load4_to_lds(thr_base, prow * 4u, thr_lds0 + buf * (kBlockRows * 4) + wave * 256);
+      const uint32_t prow = item_first_row(blk * kBlockItems + r / STEP) + (uint32_t)(r % STEP);
+      sel_load4_to_lds(thr_base, prow * 4u, thr_lds0 + buf * (ROWS * 4) + wave * 256);
     }
   };
 
@@ -224,14 +235,13 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
   typedef __attribute__((address_space(3))) floatx4 lds_floatx4_t;
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-  constexpr int kBlockItems = kGroups * kItems;  // items per block (8 or 4): lane i < kBlockItems stores item i's words
   for (int blk = 0; blk < n_blocks; ++blk) {
     const int buf = blk & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of block blk has landed
     __syncthreads();                                   // ... and everyone's; everyone is done with the other buffer
     if (blk + 1 < n_blocks) stage_block(blk + 1, buf ^ 1);
-    const uint32_t a_off = buf * (kBlockRows * kSelRowBytes);
-    // The four groups are straight-line code (no branch between them), so that the operand reads of one group can
+    const uint32_t a_off = buf * (ROWS * kSelRowBytes);
+    // The groups of a block are straight-line code (no branch between them), so that the operand reads of one group can
     // overlap the products of the previous one.  Every item is computed, also the few that cannot select this wave's
     // keys (a big block below the tile's first one, the padding past the last item): those are simply not stored.
     // The mask words of item i (wave-uniform ballot results) are dropped into lane i of w_lo / w_hi.
@@ -245,7 +255,7 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
       float thr[16];
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        const floatx4 w = *(const lds_floatx4_t*)(uintptr_t)(thr_lds0 + buf * (kBlockRows * 4) + (32 * gi + 8 * rq + 4 * half) * 4);
+        const floatx4 w = *(const lds_floatx4_t*)(uintptr_t)(thr_lds0 + buf * (ROWS * 4) + (32 * gi + 8 * rq + 4 * half) * 4);
         thr[4 * rq + 0] = w[0]; thr[4 * rq + 1] = w[1];
         thr[4 * rq + 2] = w[2]; thr[4 * rq + 3] = w[3];
       }
@@ -288,10 +298,11 @@ __global__ void __launch_bounds__(256, 2) select_scores_kernel(const SelectArgs 
 }
 
 hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
+  constexpr int kWaves = AA_SEL_WAVES, kRows = AA_SEL_ROWS;
   const int step = a.big_block / a.block_size;
-  const dim3 grid((uint32_t)(a.n_ctx / (128 * kKB)) * a.n_kv_heads * a.batch);
-  if (step == 16) hipLaunchKernelGGL(select_scores_kernel<16>, grid, dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL(select_scores_kernel<32>, grid, dim3(256), 0, stream, a);
+  const dim3 grid((uint32_t)(a.n_ctx / (64 * kWaves)) * a.n_kv_heads * a.batch);
+  if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows>), grid, dim3(64 * kWaves), 0, stream, a);
+  else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows>), grid, dim3(64 * kWaves), 0, stream, a);
   return hipGetLastError();
 }
 
