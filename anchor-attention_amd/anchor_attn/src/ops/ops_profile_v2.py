@@ -31,17 +31,19 @@ def record_recall_ratios(out: torch.Tensor, ref: torch.Tensor, sparsity_ratio, t
     return {"sparsity_ratio": float(sparsity_ratio), **{f"recall@{t}": recall_ratio(out, ref, t) for t in thresholds}}
 
 
-def theta_sweep(q, k, v, thetas: Iterable[float], block_size: int = 128, step: int = 16, ref: torch.Tensor = None) -> List[Dict]:
-    """One row per theta: sparsity ratio, error against dense attention (max / mean / recall), time per call."""
+def theta_sweep(q, k, v, thetas: Iterable[float], block_size: int = 128, step: int = 16, ref: torch.Tensor = None,
+                strict_reference: bool = True) -> List[Dict]:
+    """One row per theta: sparsity ratio, error against dense attention (max / mean / recall), time per call.
+    ``strict_reference=False`` sweeps the intended-geometry mode of the operator (analysis only)."""
     if ref is None:
         ref = dense_causal_attention(q, k, v)
     rows = []
     out = torch.empty_like(q)
     for theta in thetas:
-        anchor_attn(q, k, v, block_size=block_size, step=step, difference=theta, out=out)  # warm-up
+        anchor_attn(q, k, v, block_size=block_size, step=step, difference=theta, out=out, strict_reference=strict_reference)  # warm-up
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        _, ratio = anchor_attn(q, k, v, block_size=block_size, step=step, difference=theta, out=out)
+        _, ratio = anchor_attn(q, k, v, block_size=block_size, step=step, difference=theta, out=out, strict_reference=strict_reference)
         e1.record()
         torch.cuda.synchronize()
         mean_err, strict, loose, metrics = get_deff(ref, out, verbose=False)

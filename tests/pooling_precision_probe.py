@@ -8,7 +8,10 @@ float32 (ascending row order).  This script measures, on one workload, what the 
 it pools with an own Triton micro-kernel written like the reference's lines, feeds those pooled queries to the
 library's stage 2 (the C ABI takes them as an input) and compares index lists and final outputs.
 
-    python tests/pooling_precision_sensitivity.py [--workload config2_llama8b_128k]      (needs a GPU and Triton)
+    python tests/pooling_precision_probe.py [--workload config2_llama8b_128k]      (needs a GPU and Triton)
+
+One JSON line comes out; tests/test_gpu_parity.py::test_pooling_precision_reading_is_immaterial runs this file in a
+process of its own and asserts on that line.
 """
 import argparse
 import json
@@ -80,12 +83,14 @@ def main():
             changed += int((hot != 0).sum())
     d = (qbar.float() - qbar_t.float()).abs()
     err = (out0.float() - out1.float()).abs()
+    big = torch.maximum(out0.float().abs().max(), out1.float().abs().max())
     print(json.dumps({
         "workload": args.workload, "theta": args.theta, "triton": triton.__version__,
         "pooled_query_elements_differing": float((d != 0).float().mean()), "pooled_query_max_abs_diff": float(d.max()),
         "selected_float32_pooling": int(n0.sum()), "selected_triton_pooling": int(n1.sum()),
         "indices_in_one_list_only": changed, "fraction_of_selected": changed / max(int(n0.sum()), 1),
         "output_max_abs_diff": float(err.max()), "output_mean_abs_diff": float(err.mean()),
+        "output_max_abs": float(big),
     }))
 
 

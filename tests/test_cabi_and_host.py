@@ -172,3 +172,18 @@ def test_analysis_tools_on_cpu():
     s = (q @ k.repeat_interleave(2, 1).transpose(-1, -2)).masked_fill(torch.triu(torch.ones(70, 70, dtype=torch.bool), 1), float("-inf"))
     want = torch.gather(v.repeat_interleave(2, 1), 2, s.argmax(-1, keepdim=True).expand(-1, -1, -1, 16))
     assert torch.allclose(out0, want, atol=1e-5) and abs(r0 - 70 / (70 * 71 / 2)) < 1e-9
+
+
+def test_recall_bookkeeping_on_cpu():
+    """recall@t = fraction of elements with |out - ref| < t (strict), reported next to the sparsity ratio
+    (counterpart of the reference's ops_profile_v2.py:514-532)."""
+    from anchor_attn.src.ops.ops_profile_v2 import RECALL_THRESHOLDS, recall_ratio, record_recall_ratios
+    ref = torch.zeros(2, 5)
+    out = torch.tensor([[0.0, 0.004, 0.005, 0.0099, 0.01], [0.02, -0.004, -0.0051, 1.0, -0.0]])
+    assert recall_ratio(out, ref, 0.01) == 7 / 10     # 0.01 and 0.02 and 1.0 are not below 0.01
+    assert recall_ratio(out, ref, 0.005) == 4 / 10    # 0, 0.004, -0.004, -0 only (0.005 itself is not below)
+    assert recall_ratio(out.to(torch.bfloat16), ref, 1e9) == 1.0 and recall_ratio(out, ref, 0.0) == 0.0
+    row = record_recall_ratios(out, ref, torch.tensor(0.25))
+    assert RECALL_THRESHOLDS == (0.01, 0.005)
+    assert row == {"sparsity_ratio": 0.25, "recall@0.01": 0.7, "recall@0.005": 0.4}
+    assert record_recall_ratios(out, out, 0.5, thresholds=(1e-6,)) == {"sparsity_ratio": 0.5, "recall@1e-06": 1.0}
