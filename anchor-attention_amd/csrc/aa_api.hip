@@ -210,13 +210,13 @@ size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int
   return carve(batch, n_q_heads, n_ctx, block_size, step).total;
 }
 
-int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
-                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
-                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
-                         float* M, float* L, float* acc_frag,
-                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                         int block_size, int step, float sm_scale, int scale_mode, void* stream) {
-  const char* who = "aa_stage1_anchor_fwd";
+// Stage 1; with qbar/abar non-null (block_size <= 128) the kernel also emits the pooled queries and anchors.
+static int stage1_impl(const char* who, const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                       const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                       const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                       float* M, float* L, float* acc_frag, void* qbar, void* abar,
+                       int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                       int block_size, int step, float sm_scale, int scale_mode, void* stream) {
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
@@ -232,10 +232,21 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
   a.M_out = M; a.L_out = L; a.acc_out = acc_frag;
+  a.qbar_out = (__bf16*)qbar; a.abar_out = (__bf16*)abar;
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = scale_mode;
   return check_launch(run_flash(a, 0, (hipStream_t)stream), who);
+}
+
+int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         float* M, float* L, float* acc_frag,
+                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
+                         int block_size, int step, float sm_scale, int scale_mode, void* stream) {
+  return stage1_impl("aa_stage1_anchor_fwd", q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc_frag, nullptr,
+                     nullptr, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, scale_mode, stream);
 }
 
 int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
@@ -373,10 +384,16 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   uint32_t* mask = (uint32_t*)(ws + w.mask);
   int32_t* coords = (int32_t*)(ws + w.coords);
   int32_t* counts = (int32_t*)(ws + w.counts);
-  if ((rc = aa_stage1_anchor_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc, batch, n_q_heads,
-                                 n_kv_heads, n_ctx, head_dim, block_size, step, (float)sm_scale, scale_mode, stream)))
+  // A stage-1 work-group holds 128 query rows: whole pooled rows when block_size <= 128, and then it pools them itself
+  // (same arithmetic as aa_pool_q_anchor, bit for bit) instead of a separate pass over the queries.
+  const bool fused_pool = block_size <= 128;
+  if ((rc = stage1_impl(who, q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc, fused_pool ? qbar : nullptr,
+                        fused_pool ? abar : nullptr, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step,
+                        (float)sm_scale, scale_mode, stream)))
     return rc;
-  if ((rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, stream))) return rc;
+  if (!fused_pool &&
+      (rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, stream)))
+    return rc;
   if ((rc = aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, mask, coords, counts, batch, n_q_heads, n_kv_heads, n_ctx,
                              head_dim, block_size, step, sm_scale, theta_log2, geometry, stream)))
     return rc;

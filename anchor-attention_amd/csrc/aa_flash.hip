@@ -153,8 +153,32 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
   const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
 
+  // ---- sparse mode: the resume state and the queries are requested first --------------------------
+  // They depend on nothing, whereas the first K/V tile needs the index list, which needs its own round trip to
+  // memory: issued up front, the 100 KB of state travel while the list is fetched instead of after it.
+  u32x4 qraw[8];
+  float m_run, l_run;
+  floatx16 acc[4];
+  const __bf16* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
+  if (MODE == kSparse) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
+    m_run = p.M[bh * p.n_ctx + my_row];
+    l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
+    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
+      }
+  }
+
   // ---- tile schedule -------------------------------------------------------------------------
-  int n_tiles, n_init = 0, cnt = 0;
+  const bool pool = MODE == kAnchor && p.qbar_out != nullptr;
+  int n_tiles, n_init = 0, cnt = 0, cap = 0;
   const int32_t* cbase = nullptr;
   if (MODE == kAnchor) {
     n_init = min(S, R0 + BM) / kBN;
@@ -163,23 +187,27 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     n_tiles = (R0 + BM) / kBN;
   } else {
     cnt = p.counts[bh * (p.n_ctx / S) + bb];
+    cap = max(bb * S - 2 * p.block_size, 0);  // capacity of the big block's list (a multiple of 4)
     cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
     n_tiles = (cnt + kBN - 1) / kBN;
   }
   // first key (anchor, dense) or first list position (sparse) of tile i
 #define AA_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
 
-  // sparse mode: list positions [w0, w0 + kIdxWin) -> LDS (zeros past the count)
+  // sparse mode: list positions [w0, w0 + kIdxWin) -> LDS (zeros past the count).  The load is bounded by the list's
+  // capacity, not by its count, so that it does not have to wait for the count to arrive; what lies past the count is
+  // zeroed afterwards.
   auto fill_index_window = [&](const int w0) {
     const int pos = w0 + 4 * tid;
     int4 v = {0, 0, 0, 0};
-    if (pos < cnt) v = *reinterpret_cast<const int4*>(cbase + pos);  // lists start 16-byte aligned; capacity is a multiple of 4
+    if (pos < cap) v = *reinterpret_cast<const int4*>(cbase + pos);  // lists start 16-byte aligned; capacity is a multiple of 4
+    if (pos >= cnt) v.x = 0;
     if (pos + 1 >= cnt) v.y = 0;
     if (pos + 2 >= cnt) v.z = 0;
     if (pos + 3 >= cnt) v.w = 0;
     *reinterpret_cast<int4*>(&sm.idx[4 * tid]) = v;
   };
-  if (MODE == kSparse && n_tiles > 0) {
+  if (MODE == kSparse && cap > 0) {  // (uniform over the work-group; not conditioned on the count, see above)
     fill_index_window(0);
     __syncthreads();
   }
@@ -194,6 +222,10 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     k_voff[j] = ((tid >> 4) + 16 * j) * k_row_bytes + k_col;
     v_voff[j] = ((tid >> 4) + 16 * j) * v_row_bytes + v_col;
   }
+  // (anchor mode with pooling) the work-group's raw query rows, fetched like a tile by the last tile's load slots
+  const char* qblock = reinterpret_cast<const char*>(qp + (int64_t)R0 * p.q_sn);
+  const uint32_t q_row_bytes = (uint32_t)p.q_sn * 2u;
+  const uint32_t q_voff = (uint32_t)(tid >> 4) * q_row_bytes + (uint32_t)(tid & 15) * 16u;
   if (n_tiles > 0) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
@@ -205,27 +237,16 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   bf16x8 qreg[8];
   {
     const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
-    const __bf16* row = qp + (int64_t)my_row * p.q_sn + 8 * half;
+    if (MODE != kSparse) {
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8(*reinterpret_cast<const u32x4*>(row + 16 * ks), p.sm_scale, chain);
+      for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8(qraw[ks], p.sm_scale, chain);
   }
 
-  // ---- running state -------------------------------------------------------------------------
-  float m_run, l_run;
-  floatx16 acc[4];
-  if (MODE == kSparse) {
-    m_run = p.M[bh * p.n_ctx + my_row];
-    l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
-    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
-      }
-  } else {
+  // ---- running state (sparse mode loaded it at the top) -----------------------------------------
+  if (MODE != kSparse) {
     m_run = -INFINITY;
     l_run = 0.f;
 #pragma unroll
@@ -322,12 +343,25 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // Tile i+1 goes straight into the other buffer (every wave finished reading it before the last barrier).  Its
     // eight load instructions are spread over the first MFMAs of this tile: issued in one burst by all four waves
     // they queue up behind each other in the memory pipeline and every wave stalls for the length of the queue.
-    // (the last tile fetches itself once more into the idle buffer, which keeps the instruction stream free of branches)
+    // (the last tile fetches itself once more into the idle buffer, which keeps the instruction stream free of branches -
+    // unless the work-group also pools its queries: then the eight load slots of the last tile bring the work-group's
+    // 128 raw query rows into the idle buffer instead, rows 0..63 where K tiles go and rows 64..127 where V tiles go,
+    // chunks in place)
     const int i_next = i + 1 < n_tiles ? i + 1 : i;
     const int key0_next = AA_TILE_KEY0(i_next);
+    const bool fetch_queries = MODE == kAnchor && pool && i + 1 == n_tiles;  // wave-uniform
 #define AA_FETCH_ONE(n)                                                                                               \
-  tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,   \
-                                  lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes, k_voff, v_voff);
+  if (MODE == kAnchor) { /* selects, not branches: the eight slots stay straight-line code */                        \
+    const int j_ = (n) >> 1;                                                                                          \
+    const char* kv_ = ((n) & 1) ? vbase + (uint64_t)(uint32_t)key0_next * v_row_bytes                                 \
+                                : kbase + (uint64_t)(uint32_t)key0_next * k_row_bytes;                                \
+    const char* q_ = qblock + (uint64_t)(64 * ((n) & 1) + 16 * j_) * q_row_bytes;                                     \
+    load16_to_lds(fetch_queries ? q_ : kv_, fetch_queries ? q_voff : (((n) & 1) ? v_voff[j_] : k_voff[j_]),           \
+                  (((n) & 1) ? lds_v0 : lds_k0) + (buf ^ 1) * kTileBytes + 16 * j_ * kRowBytes);                      \
+  } else {                                                                                                            \
+    tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,             \
+                         lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes, k_voff, v_voff);           \
+  }
     // (a wave whose rows all lie above this tile - two of the four waves on the last tile of a causal work-group -
     // runs it fully masked: it would only wait at the barrier for the others anyway)
     {
@@ -505,6 +539,46 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         for (int c = 0; c < 4; ++c) t[c] = acc[db][rg * 4 + c];
         *reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256) = t;
       }
+    if (pool) {
+      // Mean-pooling of the work-group's raw queries (brought into the idle tile buffer by the last tile's load slots) and
+      // of its anchors: float32 sums over block_size rows in ascending row order, divided by block_size, rounded to
+      // bf16 - the same operations in the same order as pool_kernel, so the results are the same bit for bit.
+      const int pbuf = n_tiles & 1;  // where the queries went
+      float* mlds = reinterpret_cast<float*>(sm.t.k[pbuf ^ 1]);
+      if (half == 0) mlds[wave * 32 + c32] = m_run;
+      __syncthreads();
+      const int bs = p.block_size, n_pooled = BM / bs;  // pooled rows of this work-group (1 for block_size 128)
+      const int n_pr = p.n_ctx / bs;
+      const float d = (float)bs;
+      if (tid < 128) {
+        // waves 0 and 1: one head-dim column per thread (the ordered sum is a serial chain per column, so the shorter
+        // the chain per thread the sooner the work-group retires)
+        for (int pp = 0; pp < n_pooled; ++pp) {
+          float a0 = 0.f;
+          for (int r0 = pp * bs; r0 < (pp + 1) * bs; r0 += 16) {  // 16 rows at a time (never across the K/V halves): reads first, then the ordered sums
+            const char* rowp = (r0 < 64 ? sm.t.k[pbuf] : sm.t.v[pbuf]) + (r0 & 63) * kRowBytes + 2 * tid;
+            uint16_t w[16];
+#pragma unroll
+            for (int t = 0; t < 16; ++t) w[t] = *reinterpret_cast<const uint16_t*>(rowp + t * kRowBytes);
+#pragma unroll
+            for (int t = 0; t < 16; ++t) a0 += bf16_lo(w[t]);
+          }
+          reinterpret_cast<uint16_t*>(p.qbar_out)[((bh * n_pr) + R0 / bs + pp) * 128 + tid] = (uint16_t)(pack_bf16(a0 / d, 0.f) & 0xffffu);
+        }
+      } else if (tid - 128 < n_pooled) {
+        // meanwhile, in wave 2: one thread per pooled anchor
+        const int pp = tid - 128;
+        float am = 0.f;
+        for (int r0 = pp * bs; r0 < (pp + 1) * bs; r0 += 16) {
+          float w[16];
+#pragma unroll
+          for (int t = 0; t < 16; t += 4) *reinterpret_cast<floatx4*>(&w[t]) = *reinterpret_cast<const floatx4*>(&mlds[r0 + t]);
+#pragma unroll
+          for (int t = 0; t < 16; ++t) am += w[t];
+        }
+        reinterpret_cast<uint16_t*>(p.abar_out)[bh * n_pr + R0 / bs + pp] = (uint16_t)(pack_bf16(am / d, 0.f) & 0xffffu);
+      }
+    }
   } else {
     // out = bf16(acc / l): stage the wave's [32][128] tile in LDS, then write whole rows
     __bf16* os = sm.os[wave];

@@ -10,6 +10,9 @@ struct FlashArgs {
   const __bf16* v; int64_t v_sb, v_sh, v_sn;
   __bf16* out;     int64_t o_sb, o_sh, o_sn;   // sparse / dense modes
   float* M_out; float* L_out; float* acc_out;  // anchor mode
+  // anchor mode, optional (both or neither; block_size <= 128): the work-group also mean-pools its 128 raw query rows
+  // and anchors into qbar [B,Hq,N/block_size,128] and abar [B,Hq,N/block_size], bit for bit what pool_kernel computes
+  __bf16* qbar_out; __bf16* abar_out;
   const float* M; const float* L; const float* acc_frag;  // sparse mode (resume state)
   const int32_t* coords; const int32_t* counts; int64_t coords_per_head;  // sparse mode
   int batch, n_q_heads, n_kv_heads, n_ctx;
