@@ -132,26 +132,33 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const int c32 = lane & 31;
 
   // ---- which rows ----------------------------------------------------------------------------
+  // A work-group owns 128 query rows - in sparse mode p.q_blocks_per_wg consecutive blocks of 128 rows of one big
+  // block, one after the other: they share the big block's index list (fetched once), and the output stores of one
+  // block drain while the next one is already loading, instead of every 128 rows paying for a work-group launch, the
+  // list's round trip to memory and the wait for its stores.
   const int group = p.n_q_heads / p.n_kv_heads;
-  const int n_qblk = p.n_ctx / BM;
-  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qblk, group);
+  const int nq = MODE == kSparse ? p.q_blocks_per_wg : 1;
+  const int n_qunit = p.n_ctx / (BM * nq);
+  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qunit, group);
   const int g = vid % group;  vid /= group;
-  int qblk = vid % n_qblk;    vid /= n_qblk;
+  int qunit = vid % n_qunit;  vid /= n_qunit;
   const int kvh = vid % p.n_kv_heads;
   const int b = vid / p.n_kv_heads;
   const int hq = kvh * group + g;
-  qblk = n_qblk - 1 - qblk;  // longest rows first (later big blocks also carry the longest index lists)
-  const int R0 = qblk * BM;
+  qunit = n_qunit - 1 - qunit;  // longest rows first (later big blocks also carry the longest index lists)
   const int S = p.big_block;
-  const int bb = R0 / S;
-  const int wr0 = R0 + wave * 32;
-  const int my_row = wr0 + c32;
+  const int bb = qunit * nq * BM / S;  // (all blocks of a work-group lie in one big block: the host picks q_blocks_per_wg so)
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 
   const __bf16* qp = p.q + b * p.q_sb + hq * p.q_sh;
   const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
   const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
   const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
+
+  for (int qb = 0; qb < nq; ++qb) {
+  const int R0 = (qunit * nq + qb) * BM;
+  const int wr0 = R0 + wave * 32;
+  const int my_row = wr0 + c32;
 
   // ---- sparse mode: the resume state and the queries are requested first --------------------------
   // They depend on nothing, whereas the first K/V tile needs the index list, which needs its own round trip to
@@ -207,7 +214,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     if (pos + 3 >= cnt) v.w = 0;
     *reinterpret_cast<int4*>(&sm.idx[4 * tid]) = v;
   };
-  if (MODE == kSparse && cap > 0) {  // (uniform over the work-group; not conditioned on the count, see above)
+  // (uniform over the work-group; not conditioned on the count, see above.  Later blocks of the work-group find the
+  // list's first window still in place unless the list is longer than the window)
+  if (MODE == kSparse && cap > 0 && (qb == 0 || n_tiles > kIdxWin / kBN)) {
     fill_index_window(0);
     __syncthreads();
   }
@@ -601,11 +610,24 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       *reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c) = w;
     }
   }
+  // the staging rows just read lie where the next block's first tile is about to land
+  if (MODE == kSparse && qb + 1 < nq) __syncthreads();
+  }  // query blocks of the work-group
 }
 
+#ifndef AA_SPARSE_QBLOCKS
+#define AA_SPARSE_QBLOCKS 4  // 128-row query blocks a stage-3 work-group handles one after the other (when the big block allows)
+#endif
+
 template <int MODE>
-static hipError_t launch(const FlashArgs& a, hipStream_t stream) {
-  const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / 128);
+static hipError_t launch(const FlashArgs& args, hipStream_t stream) {
+  FlashArgs a = args;
+  a.q_blocks_per_wg = 1;
+  if (MODE == kSparse) {
+    const int per_big_block = a.big_block / 128;  // even for every supported geometry
+    a.q_blocks_per_wg = per_big_block % AA_SPARSE_QBLOCKS == 0 ? AA_SPARSE_QBLOCKS : (per_big_block % 2 == 0 ? 2 : 1);
+  }
+  const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / (128 * a.q_blocks_per_wg));
   hipLaunchKernelGGL((flash_kernel<MODE>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }

@@ -18,6 +18,7 @@ struct FlashArgs {
   int batch, n_q_heads, n_kv_heads, n_ctx;
   int big_block, block_size;
   float sm_scale; int scale_mode;
+  int q_blocks_per_wg;  // set by the launcher
 };
 
 // mode: 0 anchor (stage 1), 1 sparse (stage 3), 2 dense causal
