@@ -160,9 +160,10 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const int wr0 = R0 + wave * 32;
   const int my_row = wr0 + c32;
 
-  // ---- sparse mode: the resume state and the queries are requested first --------------------------
+  // ---- sparse mode: the queries and the softmax statistics are requested first ----------------------
   // They depend on nothing, whereas the first K/V tile needs the index list, which needs its own round trip to
-  // memory: issued up front, the 100 KB of state travel while the list is fetched instead of after it.
+  // memory.  The 64 KB of accumulator state follow the first tile's loads (further down) and are not waited for
+  // before the first scores are computed.
   u32x4 qraw[8];
   float m_run, l_run;
   floatx16 acc[4];
@@ -172,15 +173,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
     m_run = p.M[bh * p.n_ctx + my_row];
     l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
-    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
-      }
   }
 
   // ---- tile schedule -------------------------------------------------------------------------
@@ -241,6 +233,18 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0,
                            k_voff, v_voff);
   }
+  if (MODE == kSparse) {
+    // the accumulator state: the youngest loads in flight, first needed by the first P.V product
+    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
+      }
+  }
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
   bf16x8 qreg[8];
@@ -271,8 +275,16 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) negm[r] = -m_ref;
 
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
-  __syncthreads();
+  if (MODE == kSparse) {
+    // Loads complete in order and 64 registers take at least 16 load instructions, so "at most 16 outstanding" means:
+    // everything requested before the accumulator state - queries, statistics, tile 0 - has arrived.  The state
+    // itself may still be on its way while the first scores are computed (the compiler waits where it is first used).
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    lds_barrier();  // a barrier that does not wait for the loads still in flight
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
+    __syncthreads();
+  }
 
   // per-lane LDS byte offsets.  K: row c32 (+32*kb), chunk 2*ks + half, swizzled with the row's low four bits.
   // (absolute LDS addresses into the current buffer; the 32-key half and the row steps are immediate offsets)
