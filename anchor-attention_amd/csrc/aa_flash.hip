@@ -234,13 +234,15 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
                            k_voff, v_voff);
   }
   if (MODE == kSparse) {
-    // the accumulator state: the youngest loads in flight, first needed by the first P.V product
+    // the accumulator state: the youngest loads in flight, first needed by the first P.V product.  (The accumulator
+    // state and the output are touched once each: they are written and read with the non-temporal hint, so that they
+    // do not push K/V rows, which many work-groups share, out of the L2.)
     const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        const floatx4 t = *reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256);
+        const floatx4 t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256));
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
       }
@@ -558,7 +560,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         floatx4 t;
 #pragma unroll
         for (int c = 0; c < 4; ++c) t[c] = acc[db][rg * 4 + c];
-        *reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256) = t;
+        __builtin_nontemporal_store(t, reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256));
       }
     if (pool) {
       // Mean-pooling of the work-group's raw queries (brought into the idle tile buffer by the last tile's load slots) and
@@ -619,7 +621,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     for (int it = 0; it < 8; ++it) {
       const int r = it * 4 + (lane >> 4), c = lane & 15;
       const u32x4 w = *reinterpret_cast<const u32x4*>(&os[r * kOsStride + 8 * c]);
-      *reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c) = w;
+      __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c));
     }
   }
   // the staging rows just read lie where the next block's first tile is about to land
