@@ -252,6 +252,53 @@ def test_stage3_multiplicity_closed_form(small):
     assert (sel & wmask).any()
 
 
+@pytest.mark.parametrize("bs,step,n_bb", [(16, 16, 5), (32, 32, 3), (64, 16, 4), (256, 16, 2)])
+def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
+    """block_size is a parameter of all three stages (pooling width, candidate range [bs, bb*S - bs), big block
+    S = bs*step, window [0,S) U [bb*S, r]).  Independent route for every block size the reference's assert admits:
+    float64 window/selection masks and the multiplicity closed form for the output, torch bf16 casts and float64 dots
+    for the selection - none of it shares code with the oracle's tile loops."""
+    S_ = bs * step
+    N = n_bb * S_
+    q, k, v, _ = make_qkv(N, 2, 1, n_stripes=max(8, N // 64), seed=300 + bs)
+    Q, K, V = _np(q, k, v)
+    theta = 12.0
+    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta)
+    assert res.counts[:, :, 0].sum() == 0 and res.counts.sum() > 0
+    r = np.arange(N)[:, None]
+    j = np.arange(N)[None, :]
+    bb_r = r // S_
+    wmask = (j <= r) & ((j < S_) | (j >= bb_r * S_))
+    k64, v64 = K[0, 0].astype(np.float64), V[0, 0].astype(np.float64)
+    diff = torch.tensor(theta * ao.LOG2E, dtype=torch.float32)
+    for h in range(2):
+        # ---- selection, independently
+        qt = torch.from_numpy(Q[0, h])
+        qbar = (qt.view(N // bs, bs, D).double().sum(1) / bs).float().to(torch.bfloat16)
+        s1 = ao.q1_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        m_rows = np.where(wmask, s1, -np.inf).max(1)                       # the anchors are the windowed row maxima
+        np.testing.assert_allclose(res.M[0, h], m_rows, atol=2e-4)
+        abar = (torch.from_numpy(res.M[0, h]).view(N // bs, bs).double().sum(1) / bs).float().to(torch.bfloat16)
+        sc = ((qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (SM * ao.LOG2E)).float().to(torch.bfloat16)
+        hit = ((sc.float() + diff) >= abar.float()[:, None]).view(n_bb, step, N).any(1)
+        sel = np.zeros((N, N), bool)
+        for bb in range(n_bb):
+            lo, hi = bs, bb * S_ - bs
+            want = (torch.nonzero(hit[bb, lo:hi])[:, 0] + lo).numpy() if hi > lo else np.zeros(0, np.int64)
+            got = res.coords[0][h][bb]
+            assert got.size == 0 or (got[0] >= lo and got[-1] < hi)
+            assert len(set(want.tolist()) ^ set(got.tolist())) <= 2          # float64 vs float32 dots at a boundary
+            sel[bb * S_:(bb + 1) * S_, got] = True
+        # ---- output: multiplicity closed form
+        s3 = ao.q3_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        a = np.where(wmask, s1, -np.inf)
+        b = np.where(sel, s3, -np.inf)
+        mx = np.maximum(a.max(1), b.max(1))
+        w = np.exp2(a - mx[:, None]) + np.exp2(b - mx[:, None])
+        err = np.abs(res.out[0, h] - (w @ v64) / w.sum(1)[:, None])
+        assert err.max() < 2e-2 and err.mean() < 1.5e-3
+
+
 def test_stage3_constant_values_give_that_value(small):
     Q, K, V, pos, res = small
     row = ao.rn16(np.linspace(-2, 2, D).astype(np.float32))
