@@ -56,7 +56,7 @@ def anchor_attention_forward(module, query: torch.Tensor, key: torch.Tensor, val
     out = torch.empty(B, N, Hq, D, dtype=query.dtype, device=query.device)  # the layout the caller reshapes
     out_bhnd = out.transpose(1, 2)
     # Prefill of a fresh sequence without padding is the case the operator is defined for.
-    sparse_ok = N > 1 and n_kv == N and attention_mask is None and N >= big and query.dtype == torch.bfloat16
+    sparse_ok = N > 1 and n_kv == N and attention_mask is None and N >= big and query.dtype in (torch.bfloat16, torch.float16)
     if not sparse_ok:
         out_bhnd.copy_(_dense(query, key, value, attention_mask, scaling, n_kv - N if attention_mask is None else None))
         return out, None
@@ -81,13 +81,13 @@ def dense_attention_forward(module, query: torch.Tensor, key: torch.Tensor, valu
     """Plain causal attention on the library's own MFMA core (``aa_dense_causal_fwd``): the dense baseline "built on
     the same kernels" that the sparse operator is compared with.  Counterpart of the reference's ``"flash"`` pattern
     (modules/patch.py:128-130 -> modules/llama/flash_attention.py, ops/flash_attn_triton.py:641-657), with the same
-    division of labour as the sparse plug: a fresh unpadded bf16 prefill goes through the kernel in multiples of
+    division of labour as the sparse plug: a fresh unpadded bf16/fp16 prefill goes through the kernel in multiples of
     128 rows, the remaining tail rows, decode steps and padded batches through the framework's dense attention."""
     B, Hq, N, D = query.shape
     n_kv = key.shape[2]
     out = torch.empty(B, N, Hq, D, dtype=query.dtype, device=query.device)
     out_bhnd = out.transpose(1, 2)
-    kernel_ok = N >= 128 and n_kv == N and attention_mask is None and query.dtype == torch.bfloat16 and query.is_cuda
+    kernel_ok = N >= 128 and n_kv == N and attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and query.is_cuda
     if not kernel_ok:
         out_bhnd.copy_(_dense(query, key, value, attention_mask, scaling, n_kv - N if attention_mask is None else None))
         return out, None

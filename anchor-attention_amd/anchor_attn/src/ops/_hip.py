@@ -14,6 +14,8 @@ AA_SCALE_BF16_CHAIN = 0
 AA_SCALE_FP32 = 1
 AA_GEOMETRY_AS_RUN = 0    # stage-2 candidates [block_size, bb*S - block_size): what the reference's operator does
 AA_GEOMETRY_INTENDED = 1  # [S, bb*S): no double-counted keys, no never-attended gap (analysis only)
+AA_DTYPE_BF16 = 0
+AA_DTYPE_F16 = 1
 AA_STATIC_SCRATCH_BYTES = 40 * 1024 * 1024  # capacity of the library's static stage-2 scratch (aa_stage2_select_static)
 
 
@@ -36,13 +38,14 @@ _SIGNATURES = {
     "aa_coords_offset": (c_int64, [c_int, c_int, c_int]),
     "aa_mask_words": (c_int64, [c_int, c_int, c_int, c_int, c_int]),
     "aa_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
-    "aa_stage1_anchor_fwd": (c_int, _T3 * 3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_float, c_int, c_void_p]),
-    "aa_pool_q_anchor": (c_int, _T3 + [c_void_p] * 3 + [c_int, c_int, c_int, c_int, c_int, c_void_p]),
-    "aa_stage2_select": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_void_p]),
-    "aa_stage2_select_static": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 2 + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_void_p]),
-    "aa_stage3_sparse_fwd": (c_int, _T3 * 3 + [c_void_p] * 5 + _T3 + _DIMS5 + [c_int, c_int, c_float, c_void_p]),
-    "aa_anchor_attn_fwd": (c_int, _T3 * 4 + [c_void_p, c_size_t, c_void_p] + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_int, c_void_p]),
-    "aa_dense_causal_fwd": (c_int, _T3 * 4 + _DIMS5 + [c_float, c_void_p]),
+    # (every compute entry point ends with: ..., int dtype, void* stream)
+    "aa_stage1_anchor_fwd": (c_int, _T3 * 3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    "aa_pool_q_anchor": (c_int, _T3 + [c_void_p] * 3 + [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "aa_stage2_select": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 3 + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_int, c_void_p]),
+    "aa_stage2_select_static": (c_int, [c_void_p, c_void_p] + _T3 + [c_void_p] * 2 + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_int, c_void_p]),
+    "aa_stage3_sparse_fwd": (c_int, _T3 * 3 + [c_void_p] * 5 + _T3 + _DIMS5 + [c_int, c_int, c_float, c_int, c_void_p]),
+    "aa_anchor_attn_fwd": (c_int, _T3 * 4 + [c_void_p, c_size_t, c_void_p] + _DIMS5 + [c_int, c_int, c_double, c_float, c_int, c_int, c_int, c_void_p]),
+    "aa_dense_causal_fwd": (c_int, _T3 * 4 + _DIMS5 + [c_float, c_int, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
@@ -72,6 +75,16 @@ def check(rc: int) -> None:
     if rc != 0:
         msg = lib().aa_last_error().decode("utf-8", "replace")
         raise AnchorAttnHipError(f"anchor_attn HIP library error {rc}: {msg}")
+
+
+def dtype_code(t) -> int:
+    """AA_DTYPE_* of a tensor; anything but bf16 and fp16 raises (the reference silently treats other types as fp16)."""
+    import torch
+    if t.dtype == torch.bfloat16:
+        return AA_DTYPE_BF16
+    if t.dtype == torch.float16:
+        return AA_DTYPE_F16
+    raise AssertionError(f"anchor_attn kernels take bf16 or fp16 tensors, not {t.dtype}")
 
 
 def t3(t):

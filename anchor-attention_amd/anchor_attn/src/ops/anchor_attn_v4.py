@@ -7,7 +7,7 @@ gfx950 kernels reached through the C ABI in ``include/anchor_attn_hip.h``.
 
 Beyond the reference: K and V may be passed with their native (un-repeated) KV heads, any
 ``[B,H,N,D]`` view with unit last stride is taken without a copy, and ``out`` may be supplied.
-There is no CPU or eager fallback - tensors must be bf16 on the GPU.
+There is no CPU or eager fallback - tensors must be bf16 (or fp16, which the reference's kernels also take) on the GPU.
 """
 from __future__ import annotations
 
@@ -59,7 +59,8 @@ def _anchor_attn(Q, K, V, sm_scale=None, block_size=64, step=16, difference=100,
     _hip.check(_hip.lib().aa_anchor_attn_fwd(
         *_hip.t3(Q), *_hip.t3(K), *_hip.t3(V), *_hip.t3(output),
         ws.data_ptr(), ws.numel(), counts.data_ptr() if counts is not None else None,
-        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), float(difference), scale_mode, int(geometry), _stream()))
+        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), float(difference), scale_mode, int(geometry),
+        _hip.dtype_code(Q), _stream()))
     if return_sparsity_ratio:
         return output, _ratio(counts, B, H, N, block_size, step)
     return output, 1.0
@@ -71,7 +72,7 @@ def _stage3(Q, K, V, coords, counts, L, M, Acc, sm_scale, block_size, step, out=
     _hip.check(_hip.lib().aa_stage3_sparse_fwd(
         *_hip.t3(Q), *_hip.t3(K), *_hip.t3(V), coords.data_ptr(), counts.data_ptr(),
         M.data_ptr(), L.data_ptr(), Acc.data_ptr(), *_hip.t3(output),
-        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), _stream()))
+        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), _hip.dtype_code(Q), _stream()))
     return output
 
 
@@ -112,7 +113,7 @@ def anchor_attn_without_anchor(Q, K, V, sm_scale: float = None, block_size: int 
 
 def anchor_attn(Q, K, V, sm_scale: float = None, block_size: int = 128, step: int = 16, difference: float = 12,
                 return_computational_ratio: bool = True, out: torch.Tensor = None, strict_reference: bool = True):
-    """Sparse prefill attention.  ``Q`` ``[B,H,N,D]`` bf16; ``K``/``V`` ``[B,H or H_kv,N,D]``;
+    """Sparse prefill attention.  ``Q`` ``[B,H,N,D]`` bf16 or fp16; ``K``/``V`` ``[B,H or H_kv,N,D]`` of the same type;
     returns ``out`` or ``(out, ratio)`` exactly like the reference.
 
     ``strict_reference=False`` (analysis only, never the default) lets stage 2 choose from ``[S, bb*S)``
@@ -166,5 +167,5 @@ def dense_causal_attention(Q, K, V, sm_scale: float = None, out: torch.Tensor = 
     sm_scale = sm_scale if sm_scale else 1.0 / (D ** 0.5)
     output = torch.empty_like(Q) if out is None else out
     _hip.check(_hip.lib().aa_dense_causal_fwd(*_hip.t3(Q), *_hip.t3(K), *_hip.t3(V), *_hip.t3(output),
-                                              B, H, K.shape[1], N, D, float(sm_scale), _stream()))
+                                              B, H, K.shape[1], N, D, float(sm_scale), _hip.dtype_code(Q), _stream()))
     return output

@@ -27,10 +27,10 @@ def _stream() -> int:
 
 def _check_inputs(Q, K, V=None):
     assert Q.is_cuda and K.is_cuda, "anchor_attn runs on the GPU only (there is no CPU path)"
-    assert Q.dtype == torch.bfloat16 and K.dtype == torch.bfloat16, "anchor_attn kernels take bf16 inputs"
+    assert Q.dtype in (torch.bfloat16, torch.float16) and K.dtype == Q.dtype, "anchor_attn kernels take bf16 or fp16 inputs (one type per call)"
     assert Q.shape[1] % K.shape[1] == 0, "number of KV heads must divide the number of query heads"
     if V is not None:
-        assert V.dtype == torch.bfloat16 and V.shape == K.shape
+        assert V.dtype == Q.dtype and V.shape == K.shape
 
 
 def anchor_attn_step_1(Q, K, V, init_cnt, local_cnt, block_size, step, B, H, N, D, sm_scale,
@@ -46,7 +46,7 @@ def anchor_attn_step_1(Q, K, V, init_cnt, local_cnt, block_size, step, B, H, N, 
     Acc = torch.empty((B, H, N, D), dtype=torch.float32, device=Q.device)
     _hip.check(_hip.lib().aa_stage1_anchor_fwd(
         *_hip.t3(Q), *_hip.t3(K), *_hip.t3(V), M.data_ptr(), L.data_ptr(), Acc.data_ptr(),
-        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), scale_mode, _stream()))
+        B, H, K.shape[1], N, D, block_size, step, float(sm_scale), scale_mode, _hip.dtype_code(Q), _stream()))
     return L, M, Acc
 
 
@@ -60,14 +60,14 @@ def acc_rows(Acc_frag: torch.Tensor) -> torch.Tensor:
 
 
 def pool_q_anchor(Q, M_buffer, block_size):
-    """bf16 mean-pooled queries ``[B,H,N/bs,D]`` and anchors ``[B,H,N/bs]`` (get_mask_test.py:75-84)."""
+    """Mean-pooled queries ``[B,H,N/bs,D]`` and anchors ``[B,H,N/bs]`` in the queries' 16-bit type (get_mask_test.py:75-84)."""
     Q = _row_major(Q)
     B, H, N, D = Q.shape
-    qbar = torch.empty((B, H, N // block_size, D), dtype=torch.bfloat16, device=Q.device)
-    abar = torch.empty((B, H, N // block_size), dtype=torch.bfloat16, device=Q.device)
+    qbar = torch.empty((B, H, N // block_size, D), dtype=Q.dtype, device=Q.device)
+    abar = torch.empty((B, H, N // block_size), dtype=Q.dtype, device=Q.device)
     M_buffer = M_buffer.reshape(B, H, N).contiguous()
     _hip.check(_hip.lib().aa_pool_q_anchor(*_hip.t3(Q), M_buffer.data_ptr(), qbar.data_ptr(), abar.data_ptr(),
-                                           B, H, N, D, block_size, _stream()))
+                                           B, H, N, D, block_size, _hip.dtype_code(Q), _stream()))
     return qbar, abar
 
 
@@ -85,7 +85,7 @@ def select_stripes_packed(Q, K, M_buffer, block_size, step, theta, B, H, N, D, s
     counts = torch.empty((B, H, n_bb, 1), dtype=torch.int32, device=Q.device)
     _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(K), mask.data_ptr(), coords.data_ptr(),
                                     counts.data_ptr(), B, H, K.shape[1], N, D, block_size, step,
-                                    float(sm_scale), float(theta), int(geometry), _stream()))
+                                    float(sm_scale), float(theta), int(geometry), _hip.dtype_code(Q), _stream()))
     return coords, counts
 
 

@@ -116,6 +116,14 @@ int check_ptr(const void* ptr, const char* who, const char* name) {
   return AA_OK;
 }
 
+int check_dtype(int dtype, const char* who) {
+  if (dtype != AA_DTYPE_BF16 && dtype != AA_DTYPE_F16) {
+    set_error("%s: dtype %d is neither AA_DTYPE_BF16 nor AA_DTYPE_F16", who, dtype);
+    return AA_EBADARG;
+  }
+  return AA_OK;
+}
+
 int check_launch(hipError_t e, const char* who) {
   if (e != hipSuccess) {
     set_error("%s: launch failed: %s", who, hipGetErrorString(e));
@@ -183,7 +191,7 @@ using namespace aa;
 
 extern "C" {
 
-int aa_version(void) { return 1; }
+int aa_version(void) { return 2; }
 
 const char* aa_last_error(void) { return g_error; }
 
@@ -216,9 +224,10 @@ static int stage1_impl(const char* who, const void* q, int64_t q_sb, int64_t q_s
                        const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                        float* M, float* L, float* acc_frag, void* qbar, void* abar,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                       int block_size, int step, float sm_scale, int scale_mode, void* stream) {
+                       int block_size, int step, float sm_scale, int scale_mode, int dtype, void* stream) {
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
+  if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
   if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
@@ -228,14 +237,14 @@ static int stage1_impl(const char* who, const void* q, int64_t q_sb, int64_t q_s
     return AA_EBADARG;
   }
   FlashArgs a = {};
-  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
-  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
-  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const uint16_t*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const uint16_t*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
   a.M_out = M; a.L_out = L; a.acc_out = acc_frag;
-  a.qbar_out = (__bf16*)qbar; a.abar_out = (__bf16*)abar;
+  a.qbar_out = (uint16_t*)qbar; a.abar_out = (uint16_t*)abar;
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
-  a.sm_scale = sm_scale; a.scale_mode = scale_mode;
+  a.sm_scale = sm_scale; a.scale_mode = scale_mode; a.dtype = dtype;
   return check_launch(run_flash(a, 0, (hipStream_t)stream), who);
 }
 
@@ -244,23 +253,24 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
                          const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                          float* M, float* L, float* acc_frag,
                          int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                         int block_size, int step, float sm_scale, int scale_mode, void* stream) {
+                         int block_size, int step, float sm_scale, int scale_mode, int dtype, void* stream) {
   return stage1_impl("aa_stage1_anchor_fwd", q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc_frag, nullptr,
-                     nullptr, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, scale_mode, stream);
+                     nullptr, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, scale_mode, dtype, stream);
 }
 
 int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
                      void* qbar, void* abar,
-                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, void* stream) {
+                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int dtype, void* stream) {
   const char* who = "aa_pool_q_anchor";
   int rc;
+  if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_dims({batch, n_q_heads, n_q_heads, n_ctx, head_dim, block_size, 16}, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar"))) return rc;
   PoolArgs a = {};
-  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
-  a.M = M; a.qbar = (__bf16*)qbar; a.abar = (__bf16*)abar;
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_ctx = n_ctx; a.block_size = block_size;
+  a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.M = M; a.qbar = (uint16_t*)qbar; a.abar = (uint16_t*)abar;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_ctx = n_ctx; a.block_size = block_size; a.dtype = dtype;
   return check_launch(launch_pool(a, (hipStream_t)stream), who);
 }
 
@@ -268,9 +278,10 @@ int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream) {
+                     int block_size, int step, double sm_scale, float theta_log2, int geometry, int dtype, void* stream) {
   const char* who = "aa_stage2_select";
   int rc;
+  if ((rc = check_dtype(dtype, who))) return rc;
   if (geometry != AA_GEOMETRY_AS_RUN && geometry != AA_GEOMETRY_INTENDED) {
     set_error("%s: geometry %d is neither AA_GEOMETRY_AS_RUN nor AA_GEOMETRY_INTENDED", who, geometry);
     return AA_EBADARG;
@@ -281,8 +292,8 @@ int aa_stage2_select(const void* qbar, const void* abar,
       (rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")))
     return rc;
   SelectArgs a = {};
-  a.qbar = (const __bf16*)qbar; a.abar = (const __bf16*)abar;
-  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.qbar = (const uint16_t*)qbar; a.abar = (const uint16_t*)abar;
+  a.k = (const uint16_t*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.mask = mask_ws; a.coords = coords; a.counts = counts;
   a.thr = reinterpret_cast<float*>(mask_ws + mask_bit_words(batch, n_q_heads, n_ctx, block_size, step));
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
@@ -290,6 +301,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.big_block = block_size * step; a.block_size = block_size;
   a.scale2 = (float)(sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
+  a.dtype = dtype;
   a.key_lo = geometry == AA_GEOMETRY_AS_RUN ? block_size : block_size * step;
   a.key_slack = geometry == AA_GEOMETRY_AS_RUN ? block_size : 0;
   // the score kernel numbers (query head of the KV group, big block) pairs with 16 bits and addresses the pooled
@@ -309,7 +321,7 @@ int aa_stage2_select_static(const void* qbar, const void* abar,
                             const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                             int32_t* coords, int32_t* counts,
                             int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                            int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream) {
+                            int block_size, int step, double sm_scale, float theta_log2, int geometry, int dtype, void* stream) {
   const char* who = "aa_stage2_select_static";
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
@@ -323,7 +335,7 @@ int aa_stage2_select_static(const void* qbar, const void* abar,
   if ((rc = static_scratch(&ws, who))) return rc;
   // from here on exactly aa_stage2_select: same checks, same kernels, the scratch pointer as an ordinary argument
   return aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, static_cast<uint32_t*>(ws), coords, counts, batch, n_q_heads,
-                          n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, theta_log2, geometry, stream);
+                          n_kv_heads, n_ctx, head_dim, block_size, step, sm_scale, theta_log2, geometry, dtype, stream);
 }
 
 int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
@@ -333,9 +345,10 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
                          const float* M, const float* L, const float* acc_frag,
                          void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                          int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                         int block_size, int step, float sm_scale, void* stream) {
+                         int block_size, int step, float sm_scale, int dtype, void* stream) {
   const char* who = "aa_stage3_sparse_fwd";
   int rc;
+  if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
@@ -345,16 +358,16 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
       (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag")))
     return rc;
   FlashArgs a = {};
-  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
-  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
-  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
-  a.out = (__bf16*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const uint16_t*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const uint16_t*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.out = (uint16_t*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
   a.M = M; a.L = L; a.acc_frag = acc_frag;
   a.coords = coords; a.counts = counts;
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = block_size * step; a.block_size = block_size;
-  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
+  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32; a.dtype = dtype;
   return check_launch(run_flash(a, 1, (hipStream_t)stream), who);
 }
 
@@ -365,7 +378,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
                        int block_size, int step, double sm_scale, float theta_log2, int scale_mode, int geometry,
-                       void* stream) {
+                       int dtype, void* stream) {
   const char* who = "aa_anchor_attn_fwd";
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
@@ -389,17 +402,17 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   const bool fused_pool = block_size <= 128;
   if ((rc = stage1_impl(who, q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, M, L, acc, fused_pool ? qbar : nullptr,
                         fused_pool ? abar : nullptr, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step,
-                        (float)sm_scale, scale_mode, stream)))
+                        (float)sm_scale, scale_mode, dtype, stream)))
     return rc;
   if (!fused_pool &&
-      (rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, stream)))
+      (rc = aa_pool_q_anchor(q, q_sb, q_sh, q_sn, M, qbar, abar, batch, n_q_heads, n_ctx, head_dim, block_size, dtype, stream)))
     return rc;
   if ((rc = aa_stage2_select(qbar, abar, k, k_sb, k_sh, k_sn, mask, coords, counts, batch, n_q_heads, n_kv_heads, n_ctx,
-                             head_dim, block_size, step, sm_scale, theta_log2, geometry, stream)))
+                             head_dim, block_size, step, sm_scale, theta_log2, geometry, dtype, stream)))
     return rc;
   if ((rc = aa_stage3_sparse_fwd(q, q_sb, q_sh, q_sn, k, k_sb, k_sh, k_sn, v, v_sb, v_sh, v_sn, coords, counts, M, L, acc, out,
                                  o_sb, o_sh, o_sn, batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step, (float)sm_scale,
-                                 stream)))
+                                 dtype, stream)))
     return rc;
   if (counts_out != nullptr) {
     const size_t bytes = (size_t)batch * n_q_heads * (n_ctx / (block_size * step)) * 4;
@@ -414,22 +427,23 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                         void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                        float sm_scale, void* stream) {
+                        float sm_scale, int dtype, void* stream) {
   const char* who = "aa_dense_causal_fwd";
   int rc;
+  if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_common_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16}, who))) return rc;
   if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
   if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
   if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
   if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, who, "out"))) return rc;
   FlashArgs a = {};
-  a.q = (const __bf16*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
-  a.k = (const __bf16*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
-  a.v = (const __bf16*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
-  a.out = (__bf16*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
+  a.k = (const uint16_t*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.v = (const uint16_t*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
+  a.out = (uint16_t*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
   a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
   a.big_block = n_ctx; a.block_size = 128;  // one "big block": bb is always 0
-  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32;
+  a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32; a.dtype = dtype;
   return check_launch(run_flash(a, 2, (hipStream_t)stream), who);
 }
 

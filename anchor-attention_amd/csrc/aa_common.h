@@ -13,18 +13,66 @@ typedef float floatx2 __attribute__((ext_vector_type(2)));
 
 constexpr float kLog2e = 1.44269504f;  // the literal the operator's definition multiplies by
 
-// ---- bf16 <-> float -------------------------------------------------------------------------
-__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+// ---- 16-bit element types --------------------------------------------------------------------
+// The operator takes bf16 tensors (what its callers use) or fp16 tensors (which the definition also admits: every
+// ".to(dtype)" of it then rounds to fp16).  A kernel is written once against one of these two descriptions of the
+// element type: unpacking a pair from a dword, round-to-nearest-even packing, and the matching MFMA.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
-// round-to-nearest-even float -> bf16, two at a time (v_cvt_pk_bf16_f32 on gfx950)
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  floatx2 f = {a, b};
-  bf16x2 h = __builtin_convertvector(f, bf16x2);
-  return *reinterpret_cast<uint32_t*>(&h);
-}
-// float -> nearest bf16 -> float
-__device__ __forceinline__ float rn16(float a) { return bf16_lo(pack_bf16(a, 0.f)); }
+struct Bf16 {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ float lo(uint32_t u) { return __uint_as_float(u << 16); }
+  static __device__ __forceinline__ float hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+  static __device__ __forceinline__ float from16(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+  // round-to-nearest-even float -> bf16, two at a time (v_cvt_pk_bf16_f32 on gfx950)
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    floatx2 f = {a, b};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    return *reinterpret_cast<uint32_t*>(&h);
+  }
+  static __device__ __forceinline__ float round(float a) { return lo(pack(a, 0.f)); }  // float -> nearest bf16 -> float
+  // (a * b).to(bf16) as the operator's definition compiles: a float32 product, then the rounding
+  static __device__ __forceinline__ float round_product(float a, float b) { return round(a * b); }
+  static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct F16 {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ float lo(uint32_t u) { return (float)(*reinterpret_cast<f16x2*>(&u))[0]; }
+  static __device__ __forceinline__ float hi(uint32_t u) { return (float)(*reinterpret_cast<f16x2*>(&u))[1]; }
+  static __device__ __forceinline__ float from16(uint16_t h) { return lo((uint32_t)h); }
+  // round-to-nearest-even float -> fp16, two at a time (v_cvt_pk_f16_f32 on gfx950); overflow gives infinity
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    floatx2 f = {a, b};
+    f16x2 h = __builtin_convertvector(f, f16x2);
+    return *reinterpret_cast<uint32_t*>(&h);
+  }
+  static __device__ __forceinline__ float round(float a) { return lo(pack(a, 0.f)); }
+  // (a * b).to(fp16) as the operator's definition compiles: ONE rounding of the exact product (the multiply and the
+  // cast become a single mixed-precision instruction).  Written out so that it does not depend on what this compiler
+  // fuses: the product is exact in double; it is brought to float32 with round-to-odd, after which the
+  // round-to-nearest-even to fp16 is the correct rounding of the exact value.
+  static __device__ __forceinline__ float round_product(float a, float b) {
+    const double d = (double)a * (double)b;
+    float f = (float)d;
+    const double back = (double)f;
+    if (back != d) {  // inexact (also: overflow to infinity)
+      uint32_t u = __float_as_uint(f);
+      if ((u & 1u) == 0u) {  // even: the odd neighbour on d's side
+        const bool negative = (u >> 31) != 0u, larger = d > back;
+        u = (negative != larger) ? u + 1u : u - 1u;
+      }
+      f = __uint_as_float(u);
+    }
+    return round(f);
+  }
+  static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -52,7 +52,6 @@ typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
-typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8;
 
 template <bool WITH_IDX>
 struct FlashSmem {
@@ -61,27 +60,31 @@ struct FlashSmem {
       char k[2][kTileBytes];
       char v[2][kTileBytes];
     } t;
-    __bf16 os[4][32 * kOsStride];  // epilogue staging, reuses the tile space
+    uint16_t os[4][32 * kOsStride];  // epilogue staging, reuses the tile space
   };
   int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
 };
 
-__device__ __forceinline__ bf16x8 scale_q8(const u32x4 raw, const float sm_scale, const bool bf16_chain) {
+// Query pre-scaling into the exp2 domain, eight elements at a time.  `chain`: both constants and both products rounded
+// to the tensors' 16-bit type (stage 1, whose definition takes sm_scale as a compile-time constant); otherwise float32
+// products and one rounding.
+template <typename T>
+__device__ __forceinline__ typename T::vec8 scale_q8(const u32x4 raw, const float sm_scale, const bool chain) {
   const uint32_t w[4] = {raw[0], raw[1], raw[2], raw[3]};
   uint32_t o[4];
-  if (bf16_chain) {  // bf16(bf16(q * bf16(sm_scale)) * bf16(log2e))
-    const float s16 = rn16(sm_scale), c16 = rn16(kLog2e);
+  if (chain) {  // r16(r16(q * r16(sm_scale)) * r16(log2e))
+    const float s16 = T::round(sm_scale), c16 = T::round(kLog2e);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float a = rn16(bf16_lo(w[i]) * s16), b = rn16(bf16_hi(w[i]) * s16);
-      o[i] = pack_bf16(a * c16, b * c16);
+      const float a = T::round(T::lo(w[i]) * s16), b = T::round(T::hi(w[i]) * s16);
+      o[i] = T::pack(a * c16, b * c16);
     }
   } else {  // float32 products, one rounding
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = pack_bf16((bf16_lo(w[i]) * sm_scale) * kLog2e, (bf16_hi(w[i]) * sm_scale) * kLog2e);
+    for (int i = 0; i < 4; ++i) o[i] = T::pack((T::lo(w[i]) * sm_scale) * kLog2e, (T::hi(w[i]) * sm_scale) * kLog2e);
   }
   const u32x4 packed = {o[0], o[1], o[2], o[3]};
-  return *reinterpret_cast<const bf16x8*>(&packed);
+  return *reinterpret_cast<const typename T::vec8*>(&packed);
 }
 
 typedef __attribute__((address_space(3))) char lds_char;
@@ -120,8 +123,10 @@ __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, cons
   }
 }
 
-template <int MODE>
+template <int MODE, typename T>
 __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
+  typedef typename T::vec8 vec8;
+  typedef __attribute__((address_space(3))) vec8 lds_vec8;
   __shared__ __attribute__((aligned(16))) FlashSmem<MODE == kSparse> sm;
   constexpr int BM = 128;
 
@@ -150,7 +155,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const int bb = qunit * nq * BM / S;  // (all blocks of a work-group lie in one big block: the host picks q_blocks_per_wg so)
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 
-  const __bf16* qp = p.q + b * p.q_sb + hq * p.q_sh;
+  const uint16_t* qp = p.q + b * p.q_sb + hq * p.q_sh;
   const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
   const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
   const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
@@ -167,7 +172,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   u32x4 qraw[8];
   float m_run, l_run;
   floatx16 acc[4];
-  const __bf16* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
+  const uint16_t* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
   if (MODE == kSparse) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
@@ -249,7 +254,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   }
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
-  bf16x8 qreg[8];
+  vec8 qreg[8];
   {
     const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
     if (MODE != kSparse) {
@@ -257,7 +262,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8(qraw[ks], p.sm_scale, chain);
+    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8<T>(qraw[ks], p.sm_scale, chain);
   }
 
   // ---- running state (sparse mode loaded it at the top) -----------------------------------------
@@ -335,8 +340,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     const float e0 = fast_exp2(sx[4 * (c) + 0]), e1 = fast_exp2(sx[4 * (c) + 1]);    \
     const float e2 = fast_exp2(sx[4 * (c) + 2]), e3 = fast_exp2(sx[4 * (c) + 3]);    \
     sum += e0; sum += e1; sum += e2; sum += e3;                                      \
-    pw[(c) >> 1][2 * ((c) & 1) + 0] = pack_bf16(e0, e1);                             \
-    pw[(c) >> 1][2 * ((c) & 1) + 1] = pack_bf16(e2, e3);                             \
+    pw[(c) >> 1][2 * ((c) & 1) + 0] = T::pack(e0, e1);                                 \
+    pw[(c) >> 1][2 * ((c) & 1) + 1] = T::pack(e2, e3);                                 \
   }
   // V operand fetch i (two transposing reads): i = (kb*2 + st)*4 + db
 #define AA_V_SRC(i) (v_rd[(i) & 3] + (uint32_t)((32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes))
@@ -349,8 +354,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   {                                                                                                    \
     typedef short shortx8 __attribute__((ext_vector_type(8)));                                         \
     const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);                \
-    acc[(i) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&av),      \
-                                                           *reinterpret_cast<const bf16x8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3], 0, 0, 0); \
+    acc[(i) & 3] = T::mfma(*reinterpret_cast<const vec8*>(&av),                                        \
+                           *reinterpret_cast<const vec8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3]);         \
   }
 #define AA_FENCE __builtin_amdgcn_sched_barrier(0)
 
@@ -389,11 +394,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // runs it fully masked: it would only wait at the barrier for the others anyway)
     {
       floatx16 s0, s1;
-      bf16x8 ka[16];            // K operand of slot n = kb*8 + ks
+      vec8 ka[16];              // K operand of slot n = kb*8 + ks
       shortx4 vlo[16], vhi[16];  // V operand of slot 16 + i, i = (kb*2 + st)*4 + db
       u32x4 pw0[2], pw1[2];      // P^T fragments (bf16 pairs) of the two halves
       float mx0, mx1, sum0 = 0.f, sum1 = 0.f, shift0 = 0.f, alpha1 = 1.f;
-#define AA_K_FETCH(t) ka[t] = *(const lds_bf16x8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(32 * ((t) >> 3) * kRowBytes))
+#define AA_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(32 * ((t) >> 3) * kRowBytes))
 
       // The 32 MFMAs of a tile are slots 0..31 (16 for S^T, 16 for O^T); the operand of slot n is fetched from
       // LDS while slot n - kDist is issued.  The scheduling fences keep that distance: left alone, the reads sink
@@ -406,7 +411,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       AA_V_FETCH(((n) - 16) & 15)                    \
     }                                                \
   }
-#define AA_S_MFMA(sx, n) sx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[n], qreg[(n) & 7], ((n) & 7) == 0 ? negm : sx, 0, 0, 0)
+#define AA_S_MFMA(sx, n) sx = T::mfma(ka[n], qreg[(n) & 7], ((n) & 7) == 0 ? negm : sx)
 #pragma unroll
       for (int n = 0; n < kDist; ++n) AA_OPERAND_FETCH(n)
       AA_FENCE;
@@ -584,9 +589,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
             for (int t = 0; t < 16; ++t) w[t] = *reinterpret_cast<const uint16_t*>(rowp + t * kRowBytes);
 #pragma unroll
-            for (int t = 0; t < 16; ++t) a0 += bf16_lo(w[t]);
+            for (int t = 0; t < 16; ++t) a0 += T::from16(w[t]);
           }
-          reinterpret_cast<uint16_t*>(p.qbar_out)[((bh * n_pr) + R0 / bs + pp) * 128 + tid] = (uint16_t)(pack_bf16(a0 / d, 0.f) & 0xffffu);
+          reinterpret_cast<uint16_t*>(p.qbar_out)[((bh * n_pr) + R0 / bs + pp) * 128 + tid] = (uint16_t)(T::pack(a0 / d, 0.f) & 0xffffu);
         }
       } else if (tid - 128 < n_pooled) {
         // meanwhile, in wave 2: one thread per pooled anchor
@@ -599,24 +604,24 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
           for (int t = 0; t < 16; ++t) am += w[t];
         }
-        reinterpret_cast<uint16_t*>(p.abar_out)[bh * n_pr + R0 / bs + pp] = (uint16_t)(pack_bf16(am / d, 0.f) & 0xffffu);
+        reinterpret_cast<uint16_t*>(p.abar_out)[bh * n_pr + R0 / bs + pp] = (uint16_t)(T::pack(am / d, 0.f) & 0xffffu);
       }
     }
   } else {
     // out = bf16(acc / l): stage the wave's [32][128] tile in LDS, then write whole rows
-    __bf16* os = sm.os[wave];
+    uint16_t* os = sm.os[wave];
     const float inv = 1.0f / l_tot;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         u32x2 w;
-        w[0] = pack_bf16(acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv);
-        w[1] = pack_bf16(acc[db][rg * 4 + 2] * inv, acc[db][rg * 4 + 3] * inv);
+        w[0] = T::pack(acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv);
+        w[1] = T::pack(acc[db][rg * 4 + 2] * inv, acc[db][rg * 4 + 3] * inv);
         *reinterpret_cast<u32x2*>(&os[c32 * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
       }
     __syncthreads();
-    __bf16* op = p.out + b * p.o_sb + hq * p.o_sh;
+    uint16_t* op = p.out + b * p.o_sb + hq * p.o_sh;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
       const int r = it * 4 + (lane >> 4), c = lane & 15;
@@ -642,7 +647,8 @@ static hipError_t launch(const FlashArgs& args, hipStream_t stream) {
     a.q_blocks_per_wg = per_big_block % AA_SPARSE_QBLOCKS == 0 ? AA_SPARSE_QBLOCKS : (per_big_block % 2 == 0 ? 2 : 1);
   }
   const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / (128 * a.q_blocks_per_wg));
-  hipLaunchKernelGGL((flash_kernel<MODE>), dim3(grid), dim3(256), 0, stream, a);
+  if (a.dtype == 0) hipLaunchKernelGGL((flash_kernel<MODE, Bf16>), dim3(grid), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((flash_kernel<MODE, F16>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -23,6 +23,7 @@
 namespace aa {
 
 // ------------------------------------------------------------------------------------------------
+template <typename T>
 __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
   const int lane = threadIdx.x;
   const int c = lane & 15;
@@ -31,7 +32,7 @@ __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
   const int h = blockIdx.y, b = blockIdx.z;
   if (pr >= n_pr) return;
   const int bs = p.block_size;
-  const __bf16* base = p.q + b * p.q_sb + h * p.q_sh + (int64_t)pr * bs * p.q_sn + 8 * c;
+  const uint16_t* base = p.q + b * p.q_sb + h * p.q_sh + (int64_t)pr * bs * p.q_sn + 8 * c;
   const int64_t bh = (int64_t)b * p.n_q_heads + h;
   const float* mb = p.M + bh * p.n_ctx + (int64_t)pr * bs;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -39,55 +40,59 @@ __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
 #pragma unroll 8
   for (int t = 0; t < bs; ++t) {
     const uint4 raw = *reinterpret_cast<const uint4*>(base + (int64_t)t * p.q_sn);
-    acc[0] += bf16_lo(raw.x); acc[1] += bf16_hi(raw.x);
-    acc[2] += bf16_lo(raw.y); acc[3] += bf16_hi(raw.y);
-    acc[4] += bf16_lo(raw.z); acc[5] += bf16_hi(raw.z);
-    acc[6] += bf16_lo(raw.w); acc[7] += bf16_hi(raw.w);
+    acc[0] += T::lo(raw.x); acc[1] += T::hi(raw.x);
+    acc[2] += T::lo(raw.y); acc[3] += T::hi(raw.y);
+    acc[4] += T::lo(raw.z); acc[5] += T::hi(raw.z);
+    acc[6] += T::lo(raw.w); acc[7] += T::hi(raw.w);
     if (c == 0) am += mb[t];
   }
   const float d = (float)bs;
   uint4 o;
-  o.x = pack_bf16(acc[0] / d, acc[1] / d);
-  o.y = pack_bf16(acc[2] / d, acc[3] / d);
-  o.z = pack_bf16(acc[4] / d, acc[5] / d);
-  o.w = pack_bf16(acc[6] / d, acc[7] / d);
+  o.x = T::pack(acc[0] / d, acc[1] / d);
+  o.y = T::pack(acc[2] / d, acc[3] / d);
+  o.z = T::pack(acc[4] / d, acc[5] / d);
+  o.w = T::pack(acc[6] / d, acc[7] / d);
   *reinterpret_cast<uint4*>(p.qbar + (bh * n_pr + pr) * 128 + 8 * c) = o;
   if (c == 0) {
-    const uint32_t w = pack_bf16(am / d, 0.f);
+    const uint32_t w = T::pack(am / d, 0.f);
     reinterpret_cast<uint16_t*>(p.abar)[bh * n_pr + pr] = (uint16_t)(w & 0xffffu);
   }
 }
 
 hipError_t launch_pool(const PoolArgs& a, hipStream_t stream) {
   const int n_pr = a.n_ctx / a.block_size;
-  hipLaunchKernelGGL(pool_kernel, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
+  if (a.dtype == 0) hipLaunchKernelGGL(pool_kernel<Bf16>, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
+  else hipLaunchKernelGGL(pool_kernel<F16>, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
   return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------------
-// Smallest float32 x with  float(bf16(x * scale2)) + theta >= anchor  (NaN if there is none).
+// Smallest float32 x with  float(round16(x * scale2)) + theta >= anchor  (NaN if there is none); round16 rounds to the
+// tensors' 16-bit type.
+template <typename T>
 __device__ __forceinline__ bool select_test(const float x, const float scale2, const float theta, const float anchor) {
-  const float sc = rn16(x * scale2);  // float32 product, then bf16
+  const float sc = T::round_product(x, scale2);  // the score as (dot * scale).to(dtype) evaluates it for this type
   return (sc + theta) >= anchor;      // float32 add and compare, non-strict
 }
 __device__ __forceinline__ float ordered_to_float(const uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);  // monotone bijection uint32 -> float32
 }
 
-__global__ void __launch_bounds__(256) select_threshold_kernel(const __bf16* __restrict__ abar, float* __restrict__ thr, const int n,
+template <typename T>
+__global__ void __launch_bounds__(256) select_threshold_kernel(const uint16_t* __restrict__ abar, float* __restrict__ thr, const int n,
                                                                 const float scale2, const float theta) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
-  const float anchor = bf16_lo(reinterpret_cast<const uint16_t*>(abar)[i]);
+  const float anchor = T::from16(abar[i]);
   // ordered keys: 0x007fffff <-> -inf, 0xff800000 <-> +inf (NaNs lie outside that range)
   uint32_t lo = 0x007fffffu, hi = 0xff800000u;
   float out;
-  if (!select_test(ordered_to_float(hi), scale2, theta, anchor)) {
+  if (!select_test<T>(ordered_to_float(hi), scale2, theta, anchor)) {
     out = __uint_as_float(0x7fc00000u);  // no float passes: NaN compares false with everything
   } else {
     while (lo < hi) {  // invariant: test(hi) is true
       const uint32_t mid = lo + ((hi - lo) >> 1);
-      if (select_test(ordered_to_float(mid), scale2, theta, anchor)) hi = mid; else lo = mid + 1;
+      if (select_test<T>(ordered_to_float(mid), scale2, theta, anchor)) hi = mid; else lo = mid + 1;
     }
     out = ordered_to_float(hi);
   }
@@ -96,7 +101,8 @@ __global__ void __launch_bounds__(256) select_threshold_kernel(const __bf16* __r
 
 hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream) {
   const int n = a.batch * a.n_q_heads * (a.n_ctx / a.block_size);
-  hipLaunchKernelGGL(select_threshold_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.abar, a.thr, n, a.scale2, a.theta_log2);
+  if (a.dtype == 0) hipLaunchKernelGGL(select_threshold_kernel<Bf16>, dim3((n + 255) / 256), dim3(256), 0, stream, a.abar, a.thr, n, a.scale2, a.theta_log2);
+  else hipLaunchKernelGGL(select_threshold_kernel<F16>, dim3((n + 255) / 256), dim3(256), 0, stream, a.abar, a.thr, n, a.scale2, a.theta_log2);
   return hipGetLastError();
 }
 
@@ -138,7 +144,7 @@ __device__ __forceinline__ void sel_load4_to_lds(const char* base, const uint32_
   asm volatile("s_nop 0\n\tglobal_load_lds_dword %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
 }
 
-template <int STEP, int WAVES, int ROWS>
+template <int STEP, int WAVES, int ROWS, typename T>
 __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(const SelectArgs p) {
   constexpr int kItems = 32 / STEP;              // items per 32-row MFMA group
   constexpr int kGroups = ROWS / 32;             // MFMA groups per block
@@ -159,7 +165,7 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   const int n_t = p.n_ctx / 128;
   const int n_super = n_t / kTilesPerWg;
   uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, n_super, 1);
-  const int T = vid % n_super;  // key super-tile (kTilesPerWg * 128 keys); ascending = heaviest first
+  const int ST = vid % n_super;  // key super-tile (kTilesPerWg * 128 keys); ascending = heaviest first
   vid /= n_super;
   const int kvh = vid % p.n_kv_heads, b = vid / p.n_kv_heads;
   const int n_pr = p.n_ctx / p.block_size;  // pooled rows per head
@@ -170,12 +176,12 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   // Key tile t (keys 128t .. 128t+127) holds candidates of big block bb iff it reaches past key_lo and starts below
   // bb*S - key_slack, i.e. bb >= (128t + key_slack) / S + 1.
   auto tile_bb_min = [&](const int t) { return 128 * t + 128 > p.key_lo ? (128 * t + p.key_slack) / S + 1 : n_bb; };
-  const int tw = kTilesPerWg * T + wave / 2;  // this wave's 128-key tile
+  const int tw = kTilesPerWg * ST + wave / 2;  // this wave's 128-key tile
   const int kb0 = kKB * (wave % 2);           // its first 32-key block inside the tile
   const int bb_min_w = tile_bb_min(tw);
   int bb_lo = n_bb;                           // smallest big block any wave of the work-group needs
 #pragma unroll
-  for (int i = 0; i < kTilesPerWg; ++i) bb_lo = min(bb_lo, tile_bb_min(kTilesPerWg * T + i));
+  for (int i = 0; i < kTilesPerWg; ++i) bb_lo = min(bb_lo, tile_bb_min(kTilesPerWg * ST + i));
   if (bb_lo >= n_bb) return;
   const int group = p.n_q_heads / p.n_kv_heads;
   const int n_items = group * (n_bb - bb_lo);
@@ -185,13 +191,14 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   const uint32_t magic = (0x80000000u + (uint32_t)group - 1u) / (uint32_t)group;
   auto item_bb_off = [&](const int item) { return (int)__umulhi(2u * (uint32_t)item, magic); };
 
-  const __bf16* kp = p.k + b * p.k_sb + kvh * p.k_sh;
-  bf16x8 kreg[kKB][8];
+  typedef typename T::vec8 vec8;
+  const uint16_t* kp = p.k + b * p.k_sb + kvh * p.k_sh;
+  vec8 kreg[kKB][8];
 #pragma unroll
   for (int kb = 0; kb < kKB; ++kb) {
-    const __bf16* row = kp + (int64_t)(tw * 128 + 32 * (kb0 + kb) + c32) * p.k_sn + 8 * half;
+    const uint16_t* row = kp + (int64_t)(tw * 128 + 32 * (kb0 + kb) + c32) * p.k_sn + 8 * half;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const bf16x8*>(row + 16 * ks);
+    for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const vec8*>(row + 16 * ks);
   }
 
   // ---- staging -------------------------------------------------------------------------------
@@ -231,7 +238,7 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   uint32_t a_rd[8];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) a_rd[ks] = sel_lds_addr(a_lds[0]) + c32 * kSelRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
-  typedef __attribute__((address_space(3))) bf16x8 lds_bf16x8_t;
+  typedef __attribute__((address_space(3))) vec8 lds_vec8_t;
   typedef __attribute__((address_space(3))) floatx4 lds_floatx4_t;
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -248,9 +255,9 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
     uint32_t w_lo = 0u, w_hi = 0u;
 #pragma unroll
     for (int gi = 0; gi < kGroups; ++gi) {
-      bf16x8 a[8];
+      vec8 a[8];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) a[ks] = *(const lds_bf16x8_t*)(uintptr_t)(a_rd[ks] + a_off + gi * 32 * kSelRowBytes);
+      for (int ks = 0; ks < 8; ++ks) a[ks] = *(const lds_vec8_t*)(uintptr_t)(a_rd[ks] + a_off + gi * 32 * kSelRowBytes);
       // raw-score thresholds of the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
       float thr[16];
 #pragma unroll
@@ -262,11 +269,11 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
       floatx16 c[kKB];
       const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kb = 0; kb < kKB; ++kb) c[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kreg[kb][0], zero, 0, 0, 0);
+      for (int kb = 0; kb < kKB; ++kb) c[kb] = T::mfma(a[0], kreg[kb][0], zero);
 #pragma unroll
       for (int ks = 1; ks < 8; ++ks)
 #pragma unroll
-        for (int kb = 0; kb < kKB; ++kb) c[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], kreg[kb][ks], c[kb], 0, 0, 0);
+        for (int kb = 0; kb < kKB; ++kb) c[kb] = T::mfma(a[ks], kreg[kb][ks], c[kb]);
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb) {
         bool hit[kItems];
@@ -301,8 +308,13 @@ hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
   constexpr int kWaves = AA_SEL_WAVES, kRows = AA_SEL_ROWS;
   const int step = a.big_block / a.block_size;
   const dim3 grid((uint32_t)(a.n_ctx / (64 * kWaves)) * a.n_kv_heads * a.batch);
-  if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows>), grid, dim3(64 * kWaves), 0, stream, a);
-  else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows>), grid, dim3(64 * kWaves), 0, stream, a);
+  if (a.dtype == 0) {
+    if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows, Bf16>), grid, dim3(64 * kWaves), 0, stream, a);
+    else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows, Bf16>), grid, dim3(64 * kWaves), 0, stream, a);
+  } else {
+    if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows, F16>), grid, dim3(64 * kWaves), 0, stream, a);
+    else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows, F16>), grid, dim3(64 * kWaves), 0, stream, a);
+  }
   return hipGetLastError();
 }
 

@@ -211,7 +211,7 @@ def main():
             counts = torch.empty((1, hq, n_ctx // S, 1), dtype=torch.int32, device=dev)
         _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(k), mask.data_ptr(), coords.data_ptr(),
                                         counts.data_ptr(), 1, hq, hkv, n_ctx, D, BS, STEP, sm, theta2, _hip.AA_GEOMETRY_AS_RUN,
-                                        torch.cuda.current_stream().cuda_stream))
+                                        _hip.AA_DTYPE_BF16, torch.cuda.current_stream().cuda_stream))
         ev[i][3].record()
         v4._stage3(q, k, v, coords, counts, L, M, Acc, sm, BS, STEP, out=out)
         ev[i][4].record()

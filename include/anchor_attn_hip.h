@@ -10,7 +10,8 @@
  * Tensors: q/out are [batch, n_q_heads, n_ctx, head_dim]; k/v are [batch, n_kv_heads, n_ctx,
  * head_dim] with n_kv_heads dividing n_q_heads (query head h reads KV head
  * h / (n_q_heads / n_kv_heads), the order repeat_kv produces; pass n_kv_heads == n_q_heads for
- * pre-repeated K/V as the reference's caller does).  Element type is bf16, head_dim must be
+ * pre-repeated K/V as the reference's caller does).  Element type is bf16 or fp16 (the `dtype`
+ * argument, AA_DTYPE_*, the same for every tensor of a call), head_dim must be
  * 128 with stride 1, every row must start on a 16-byte boundary; the other three dimensions
  * are addressed through the element strides (sb, sh, sn), so [B,N,H,D] storage works unchanged.
  * "S" below is the big block, block_size * step keys/queries.
@@ -28,14 +29,21 @@ extern "C" {
 #endif
 
 #define AA_OK 0
-#define AA_EBADARG 1      /* null pointer, non-positive size, head counts that do not divide */
-#define AA_EUNSUPPORTED 2 /* head_dim != 128, block_size != 128, step not 16/32, n_ctx % S != 0 */
+#define AA_EBADARG 1      /* null pointer, non-positive size, head counts that do not divide, unknown dtype/mode */
+#define AA_EUNSUPPORTED 2 /* head_dim != 128, block_size not in 16..256, step not 16/32, n_ctx % S != 0, n_ctx > 2^20 */
 #define AA_EMISALIGNED 3  /* pointer or stride not a multiple of 16 bytes */
 #define AA_ELAUNCH 4      /* HIP runtime error at launch */
 
+/* Element type of q, k, v, out and of the pooled queries/anchors.  The reference takes bf16 and fp16 tensors
+ * (dtype = tl.bfloat16 if Q.dtype == torch.bfloat16 else tl.float16: anchor_step_1_2_v2.py:193, anchor_attn_v4.py:265,
+ * get_mask_test.py:157); every ".to(dtype)" of its kernels - scaled queries, probabilities, pooled queries and
+ * anchors, stage-2 scores, output - then rounds to that type.  Accumulators and M, L, Acc are float32 either way. */
+#define AA_DTYPE_BF16 0
+#define AA_DTYPE_F16 1
+
 /* How stage 1 pre-scales queries.  AA_SCALE_BF16_CHAIN reproduces the reference's stage-1
  * kernel, where sm_scale is a compile-time constant and q * sm_scale * 1.44269504 is therefore
- * evaluated in bf16 with a rounding after each multiply (anchor_step_1_2_v2.py:19,115-116).
+ * evaluated in the tensors' 16-bit type with a rounding after each multiply (anchor_step_1_2_v2.py:19,115-116).
  * AA_SCALE_FP32 is the float32 product rounded once (what stage 3 does, anchor_attn_v4.py:66). */
 #define AA_SCALE_BF16_CHAIN 0
 #define AA_SCALE_FP32 1
@@ -82,20 +90,20 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
                          const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                          float* M, float* L, float* acc_frag,
                          int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                         int block_size, int step, float sm_scale, int scale_mode, void* stream);
+                         int block_size, int step, float sm_scale, int scale_mode, int dtype, void* stream);
 
 /* ---- stage 2: difference-aware stripe identification -------------------------------------- */
 
-/* Mean-pools raw queries and anchors over block_size rows, rounding to bf16
- * (get_mask_test.py:75-84): qbar [B,Hq,N/block_size,128] bf16, abar [B,Hq,N/block_size] bf16.
+/* Mean-pools raw queries and anchors over block_size rows, rounding to the 16-bit type
+ * (get_mask_test.py:75-84): qbar [B,Hq,N/block_size,128], abar [B,Hq,N/block_size], both of the tensors' 16-bit type.
  * Sums run in float32 in ascending row order. */
 int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
                      void* qbar, void* abar,
-                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, void* stream);
+                     int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int dtype, void* stream);
 
 /* Replaces anchor_attn_step_2 / get_q_mask / get_q_mask_triton (anchor_step_1_2_v2.py:199-210,
  * get_mask_test.py:7-159): key j in [block_size, bb*S - block_size) is selected for big block bb
- * iff for one of its pooled rows i  float(bf16(dot(qbar_i,k_j) * sm_scale*1.44269504)) + theta_log2
+ * iff for one of its pooled rows i  float(round16(dot(qbar_i,k_j) * sm_scale*1.44269504)) + theta_log2
  * >= float(abar_i).  theta_log2 is float32(theta * 1.44269504), the product formed in double precision as the
  * reference's entry does with Python floats (anchor_attn_v4.py:298) and handed to the kernel as a float32
  * argument.  sm_scale is a double because the score scale is a compile-time constant in the reference's kernel:
@@ -107,7 +115,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
                      const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                      uint32_t* mask_ws, int32_t* coords, int32_t* counts,
                      int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                     int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream);
+                     int block_size, int step, double sm_scale, float theta_log2, int geometry, int dtype, void* stream);
 
 /* Same operation, same kernels and same results as aa_stage2_select, for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc) and therefore cannot provide
@@ -125,12 +133,12 @@ int aa_stage2_select_static(const void* qbar, const void* abar,
                             const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                             int32_t* coords, int32_t* counts,
                             int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                            int block_size, int step, double sm_scale, float theta_log2, int geometry, void* stream);
+                            int block_size, int step, double sm_scale, float theta_log2, int geometry, int dtype, void* stream);
 
 /* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
  * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
  * :246-268): resumes the online softmax from (M, L, acc_frag) over the K/V rows gathered at the
- * big block's selected indices and writes out = bf16(acc / l).  M, L, acc_frag are read-only. */
+ * big block's selected indices and writes out = round16(acc / l).  M, L, acc_frag are read-only. */
 int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                          const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                          const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
@@ -138,7 +146,7 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
                          const float* M, const float* L, const float* acc_frag,
                          void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                          int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                         int block_size, int step, float sm_scale, void* stream);
+                         int block_size, int step, float sm_scale, int dtype, void* stream);
 
 /* ---- whole operator -------------------------------------------------------------------------
  * Replaces _anchor_attn (anchor_attn_v4.py:226-273): stage 1 -> pooling -> stage 2 -> stage 3 on
@@ -155,18 +163,18 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                        void* workspace, size_t workspace_bytes, int32_t* counts_out,
                        int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
                        int block_size, int step, double sm_scale, float theta_log2, int scale_mode, int geometry,
-                       void* stream);
+                       int dtype, void* stream);
 
 /* ---- dense causal baseline on the same MFMA core --------------------------------------------
  * Counterpart of the reference's dense comparison path (flash_attn_triton.py:83-211, GQA mapping
- * :129-132): plain causal softmax attention, out = bf16(softmax(q k^T * sm_scale) v).
+ * :129-132): plain causal softmax attention, out = round16(softmax(q k^T * sm_scale) v).
  * n_ctx must be a multiple of 128. */
 int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                         const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                         const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,
                         void* out, int64_t o_sb, int64_t o_sh, int64_t o_sn,
                         int batch, int n_q_heads, int n_kv_heads, int n_ctx, int head_dim,
-                        float sm_scale, void* stream);
+                        float sm_scale, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -27,7 +27,8 @@ requirements.txt pins 3.2.0, which is not installed here).  ``stage1_scale_mode`
 
 Conventions: ``Q`` is ``[B, Hq, N, D]``, ``K``/``V`` are ``[B, Hkv, N, D]`` with ``Hkv | Hq``
 (query head ``h`` reads KV head ``h // (Hq // Hkv)``, the order ``repeat_kv`` produces);
-all arrays are float32 holding bf16-representable values.  ``S = block_size * step`` is the
+all arrays are float32 holding values representable in the tensors' 16-bit type: bf16, the type every caller of
+the reference uses and the default of every function here, or fp16 (``dtype="fp16"``), which its kernels also take.  ``S = block_size * step`` is the
 "big block"; ``LOG2E`` is the literal 1.44269504 the reference multiplies by.
 """
 from __future__ import annotations
@@ -67,38 +68,50 @@ def f32(x) -> np.float32:
     return np.float32(x)
 
 
+def rnd16(x: np.ndarray, dtype: str = "bf16") -> np.ndarray:
+    """Round float32 to the tensors' 16-bit type and back: what a ``.to(dtype)`` of the reference's kernels does,
+    where ``dtype`` is ``tl.bfloat16`` for bf16 inputs and ``tl.float16`` otherwise (anchor_step_1_2_v2.py:193,
+    get_mask_test.py:157, anchor_attn_v4.py:265).  ``"fp16"``: IEEE half, ties to even, overflow to infinity."""
+    if dtype == "bf16":
+        return rn16(x)
+    if dtype == "fp16":
+        with np.errstate(over="ignore"):
+            return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+    raise ValueError(dtype)
+
+
 # --------------------------------------------------------------------------------------
 # query scaling chains
 # --------------------------------------------------------------------------------------
-def q1_scale_chain(q: np.ndarray, sm_scale: float, mode: str = "bf16_chain") -> np.ndarray:
+def q1_scale_chain(q: np.ndarray, sm_scale: float, mode: str = "bf16_chain", dtype: str = "bf16") -> np.ndarray:
     """Stage-1 query pre-scaling (anchor_step_1_2_v2.py:115-116).
 
     ``sm_scale`` is a compile-time constant there, so ``q * sm_scale * 1.44269504`` is
     evaluated on a bf16 tensor with both constants materialised as bf16 and a bf16 rounding
-    after each multiply (``mode="bf16_chain"``).  ``mode="fp32"`` is the alternative reading
-    (float32 products, one rounding) kept as a switch.
+    after each multiply (``mode="bf16_chain"``; with fp16 tensors the same chain runs in fp16).
+    ``mode="fp32"`` is the alternative reading (float32 products, one rounding) kept as a switch.
     """
     q = np.asarray(q, dtype=np.float32)
     if mode == "bf16_chain":
-        s = rn16(np.array([sm_scale], dtype=np.float32))[0]
-        c = rn16(np.array([LOG2E], dtype=np.float32))[0]
-        return rn16(rn16(q * s) * c)
+        s = rnd16(np.array([sm_scale], dtype=np.float32), dtype)[0]
+        c = rnd16(np.array([LOG2E], dtype=np.float32), dtype)[0]
+        return rnd16(rnd16(q * s, dtype) * c, dtype)
     if mode == "fp32":
-        return q3_scale_chain(q, sm_scale)
+        return q3_scale_chain(q, sm_scale, dtype)
     raise ValueError(mode)
 
 
-def q3_scale_chain(q: np.ndarray, sm_scale: float) -> np.ndarray:
+def q3_scale_chain(q: np.ndarray, sm_scale: float, dtype: str = "bf16") -> np.ndarray:
     """Stage-3 query pre-scaling (anchor_attn_v4.py:65-66): ``sm_scale`` is a run-time float32
     argument, so both multiplies are float32 and there is a single rounding to bf16."""
     q = np.asarray(q, dtype=np.float32)
-    return rn16((q * np.float32(sm_scale)) * np.float32(LOG2E))
+    return rnd16((q * np.float32(sm_scale)) * np.float32(LOG2E), dtype)
 
 
 # --------------------------------------------------------------------------------------
 # stage 1: anchor / window flash attention
 # --------------------------------------------------------------------------------------
-def _online_tile(m, l, acc, s, v):
+def _online_tile(m, l, acc, s, v, dtype="bf16"):
     """One online-softmax tile update in the exp2 domain (anchor_step_1_2_v2.py:130-137 and
     anchor_attn_v4.py:91-101): float32 row sum of the unrounded ``p``, bf16 ``p`` into PV."""
     m_new = np.maximum(m, s.max(axis=1))
@@ -106,7 +119,7 @@ def _online_tile(m, l, acc, s, v):
     alpha = np.exp2(m - m_new).astype(np.float32)
     l = l * alpha + p.sum(axis=1, dtype=np.float32)
     acc = acc * alpha[:, None]
-    acc = acc + rn16(p) @ v
+    acc = acc + rnd16(p, dtype) @ v
     return m_new, l, acc
 
 
@@ -119,6 +132,7 @@ def stage1_anchor(
     step: int = 16,
     scale_mode: str = "bf16_chain",
     tile_n: int = 128,
+    dtype: str = "bf16",
 ) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
     """Windowed flash attention that yields the anchors.
 
@@ -149,7 +163,7 @@ def stage1_anchor(
             for bb in range(n_bb):
                 r0 = bb * S
                 rows = np.arange(r0, r0 + S)
-                q1 = q1_scale_chain(Q[b, h, r0 : r0 + S], sm_scale, scale_mode)
+                q1 = q1_scale_chain(Q[b, h, r0 : r0 + S], sm_scale, scale_mode, dtype)
                 m = np.full(S, -np.inf, np.float32)
                 l = np.zeros(S, np.float32)
                 acc = np.zeros((S, D), np.float32)
@@ -160,7 +174,7 @@ def stage1_anchor(
                     s = q1 @ k[j : j + tile_n].T
                     keys = np.arange(j, j + tile_n)
                     s = s + np.where(keys[None, :] <= rows[:, None], np.float32(0), MASK_ADD)
-                    m, l, acc = _online_tile(m, l, acc, s.astype(np.float32), v[j : j + tile_n])
+                    m, l, acc = _online_tile(m, l, acc, s.astype(np.float32), v[j : j + tile_n], dtype)
                 M[b, h, r0 : r0 + S] = m
                 L[b, h, r0 : r0 + S] = l
                 Acc[b, h, r0 : r0 + S] = acc
@@ -189,29 +203,40 @@ def pool_rows_f32_sequential(x: np.ndarray, block: int) -> np.ndarray:
     return acc
 
 
-def pooled_queries(Qh: np.ndarray, block_size: int) -> np.ndarray:
+def pooled_queries(Qh: np.ndarray, block_size: int, dtype: str = "bf16") -> np.ndarray:
     """``rn16(mean over each 128-row block)`` of the raw (unscaled) queries of one head
     (get_mask_test.py:75-78).  ``Qh`` is ``[N, D]``; returns ``[N/block, D]``."""
     s = pool_rows_f32_sequential(Qh.astype(np.float32), block_size)
-    return rn16(s / np.float32(block_size))
+    return rnd16(s / np.float32(block_size), dtype)
 
 
-def pooled_anchors(Mh: np.ndarray, block_size: int) -> Tuple[np.ndarray, np.ndarray]:
+def pooled_anchors(Mh: np.ndarray, block_size: int, dtype: str = "bf16") -> Tuple[np.ndarray, np.ndarray]:
     """``rn16(mean over each 128-row block)`` of the anchors (get_mask_test.py:81-84).
     Returns ``(rounded, unrounded float32 mean)``; the second is only used to classify
     near-boundary disagreements in tests."""
     s = pool_rows_f32_sequential(Mh.astype(np.float32)[:, None], block_size)[:, 0]
     mean = (s / np.float32(block_size)).astype(np.float32)
-    return rn16(mean), mean
+    return rnd16(mean, dtype), mean
 
 
-def stage2_scores(qbar: np.ndarray, k_rows: np.ndarray, sm_scale: float) -> Tuple[np.ndarray, np.ndarray]:
-    """Pooled-query x key scores of get_mask_test.py:86,96-97: float32 dot, float32 multiply by
-    ``sm_scale * 1.44269504`` (a double-precision product turned into a float32 constant), then a
-    bf16 rounding.  Returns ``(rounded, pre_rounding)`` as float32 ``[rows, keys]``."""
+def stage2_scores(qbar: np.ndarray, k_rows: np.ndarray, sm_scale: float, dtype: str = "bf16") -> Tuple[np.ndarray, np.ndarray]:
+    """Pooled-query x key scores of get_mask_test.py:86,96-97: float32 dot, multiplied by
+    ``sm_scale * 1.44269504`` (a double-precision product turned into a float32 constant) and cast to the 16-bit
+    type.  Returns ``(rounded, pre_rounding)`` as float32 ``[rows, keys]``.
+
+    bf16: a float32 product, then the rounding (two roundings; pinned bit for bit by the Triton probe).
+    fp16: the Triton tool chain compiles ``(dot * scale).to(tl.float16)`` into one mixed-precision instruction that
+    rounds the exact product once (pinned bit for bit by the same probe, tests/golden/triton_scale_chain_probe_fp16.npz);
+    that is what is restated here.  It differs from two roundings only where the float32 product is exactly half-way
+    between two fp16 values."""
     scale2 = np.float32(sm_scale * LOG2E)
-    raw = ((qbar @ k_rows.T).astype(np.float32) * scale2).astype(np.float32)
-    return rn16(raw), raw
+    dot = (qbar @ k_rows.T).astype(np.float32)
+    raw = (dot * scale2).astype(np.float32)
+    if dtype == "fp16":
+        with np.errstate(over="ignore"):
+            once = (dot.astype(np.float64) * np.float64(scale2)).astype(np.float16).astype(np.float32)
+        return once, raw
+    return rnd16(raw, dtype), raw
 
 
 def stage2_select(
@@ -223,6 +248,7 @@ def stage2_select(
     block_size: int = 128,
     step: int = 16,
     strict_reference: bool = True,
+    dtype: str = "bf16",
 ) -> Tuple[List[List[List[np.ndarray]]], np.ndarray]:
     """Difference-aware stripe identification (``get_q_mask_triton``).
 
@@ -249,15 +275,15 @@ def stage2_select(
         per_b = []
         for h in range(Hq):
             k = K[b, h // group]
-            qbar = pooled_queries(Q[b, h], block_size)
-            abar, _ = pooled_anchors(M[b, h], block_size)
+            qbar = pooled_queries(Q[b, h], block_size, dtype)
+            abar, _ = pooled_anchors(M[b, h], block_size, dtype)
             per_h = []
             for bb in range(n_bb):
                 lo, hi = (block_size, bb * S - block_size) if strict_reference else (S, bb * S)
                 if hi <= lo:
                     per_h.append(np.zeros(0, np.int32))
                     continue
-                sc, _ = stage2_scores(qbar[bb * step : (bb + 1) * step], k[lo:hi], sm_scale)
+                sc, _ = stage2_scores(qbar[bb * step : (bb + 1) * step], k[lo:hi], sm_scale, dtype)
                 hit = (sc + diff) >= abar[bb * step : (bb + 1) * step, None]
                 idx = (np.nonzero(hit.any(axis=0))[0] + lo).astype(np.int32)
                 per_h.append(idx)
@@ -295,6 +321,7 @@ def stage3_sparse(
     block_size: int = 128,
     step: int = 16,
     num_indices: int = 128,
+    dtype: str = "bf16",
 ) -> np.ndarray:
     """Resume the online softmax of stage 1 over the selected keys of the row's big block
     (``_triton_stripe_sparse_attn_fwd_kernel_step3``): chunks of 128 indices, lanes beyond the
@@ -312,7 +339,7 @@ def stage3_sparse(
             v = V[b, h // group]
             for bb in range(n_bb):
                 r0 = bb * S
-                q3 = q3_scale_chain(Q[b, h, r0 : r0 + S], sm_scale)
+                q3 = q3_scale_chain(Q[b, h, r0 : r0 + S], sm_scale, dtype)
                 m = M[b, h, r0 : r0 + S].copy()
                 l = L[b, h, r0 : r0 + S].copy()
                 acc = Acc[b, h, r0 : r0 + S].copy()
@@ -326,8 +353,8 @@ def stage3_sparse(
                     if pad:
                         s = np.concatenate([s, np.full((S, pad), -np.inf, np.float32)], axis=1)
                         vv = np.concatenate([vv, np.zeros((pad, D), np.float32)], axis=0)
-                    m, l, acc = _online_tile(m, l, acc, s, vv)
-                out[b, h, r0 : r0 + S] = rn16(acc / l[:, None])
+                    m, l, acc = _online_tile(m, l, acc, s, vv, dtype)
+                out[b, h, r0 : r0 + S] = rnd16(acc / l[:, None], dtype)
     return out
 
 
@@ -361,6 +388,7 @@ def anchor_attn_reference(
     difference: float = 12.0,
     stage1_scale_mode: str = "bf16_chain",
     strict_reference: bool = True,
+    dtype: str = "bf16",
 ) -> OracleResult:
     """The operator end to end, as ``anchor_attn`` runs it (anchor_attn_v4.py:291-324)."""
     B, Hq, N, D = Q.shape
@@ -368,9 +396,9 @@ def anchor_attn_reference(
     assert N % (block_size * step) == 0
     if not sm_scale:
         sm_scale = 1.0 / math.sqrt(D)
-    M, L, Acc = stage1_anchor(Q, K, V, sm_scale, block_size, step, stage1_scale_mode)
-    coords, counts = stage2_select(Q, K, M, sm_scale, difference, block_size, step, strict_reference)
-    out = stage3_sparse(Q, K, V, coords, counts, M, L, Acc, sm_scale, block_size, step)
+    M, L, Acc = stage1_anchor(Q, K, V, sm_scale, block_size, step, stage1_scale_mode, dtype=dtype)
+    coords, counts = stage2_select(Q, K, M, sm_scale, difference, block_size, step, strict_reference, dtype=dtype)
+    out = stage3_sparse(Q, K, V, coords, counts, M, L, Acc, sm_scale, block_size, step, dtype=dtype)
     ratio = sparsity_ratio(counts, B, Hq, N, block_size, step)
     return OracleResult(out, M, L, Acc, coords, counts, ratio)
 
@@ -378,8 +406,10 @@ def anchor_attn_reference(
 # --------------------------------------------------------------------------------------
 # helpers for the index-parity rule
 # --------------------------------------------------------------------------------------
-def _bf16_step(b: float, up: bool) -> float:
-    """Next bf16 value above (``up``) or below a bf16-representable number."""
+def _bf16_step(b: float, up: bool, dtype: str = "bf16") -> float:
+    """Next value of the 16-bit type above (``up``) or below a number representable in it."""
+    if dtype == "fp16":
+        return float(np.nextafter(np.float16(b), np.float16(np.inf if up else -np.inf)))
     b = np.float32(b)
     if b == 0:
         tiny = np.array([0x00010000], np.uint32).view(np.float32)[0]
@@ -390,7 +420,7 @@ def _bf16_step(b: float, up: bool) -> float:
     return float(np.array([bits], np.uint32).view(np.float32)[0])
 
 
-def stage2_decision_boundary(abar: float, theta: float) -> float:
+def stage2_decision_boundary(abar: float, theta: float, dtype: str = "bf16") -> float:
     """The pre-rounding score at which one pooled row's stage-2 decision flips.
 
     The decision ``float32(rn16(raw) + diff) >= abar`` is monotone in ``raw``: it becomes true
@@ -398,13 +428,13 @@ def stage2_decision_boundary(abar: float, theta: float) -> float:
     ``b`` when ``raw`` crosses the midpoint between ``b`` and the bf16 value below it."""
     diff = np.float32(theta * LOG2E)
     abar = np.float32(abar)
-    b = float(rn16(np.array([np.float32(abar - diff)], np.float32))[0])
+    b = float(rnd16(np.array([np.float32(abar - diff)], np.float32), dtype)[0])
     passes = lambda c: bool(np.float32(np.float32(c) + diff) >= abar)
     while passes(b):
-        b = _bf16_step(b, up=False)
+        b = _bf16_step(b, False, dtype)
     while not passes(b):
-        b = _bf16_step(b, up=True)
-    return 0.5 * (b + _bf16_step(b, up=False))
+        b = _bf16_step(b, True, dtype)
+    return 0.5 * (b + _bf16_step(b, False, dtype))
 
 
 def stage2_flip_distance(
@@ -414,6 +444,7 @@ def stage2_flip_distance(
     k_row: np.ndarray,
     sm_scale: float,
     theta: float,
+    dtype: str = "bf16",
 ) -> float:
     """Distance (in pre-rounding score units) of one key from the nearest point at which its
     stage-2 decision would flip: the minimum over the big block's pooled rows of
@@ -421,14 +452,14 @@ def stage2_flip_distance(
     is excusable when the distance is below the parity band (1e-3).  If a pooled anchor's
     unrounded mean lies within 1e-4 of a bf16 rounding boundary the threshold itself is ambiguous
     at float32 accuracy and 0 is returned."""
-    _, raw = stage2_scores(qbar_rows, k_row[None, :], sm_scale)
+    _, raw = stage2_scores(qbar_rows, k_row[None, :], sm_scale, dtype)
     raw = raw[:, 0].astype(np.float64)
     best = np.inf
     for i in range(raw.size):
         a = float(abar_rows[i])
         mean = float(abar_mean_rows[i])
-        for nb in (_bf16_step(a, True), _bf16_step(a, False)):
+        for nb in (_bf16_step(a, True, dtype), _bf16_step(a, False, dtype)):
             if abs(mean - 0.5 * (a + nb)) < 1e-4:
                 return 0.0
-        best = min(best, abs(raw[i] - stage2_decision_boundary(a, theta)))
+        best = min(best, abs(raw[i] - stage2_decision_boundary(a, theta, dtype)))
     return float(best)

@@ -63,7 +63,7 @@ def main():
         counts = torch.empty((B, H, N // S, 1), dtype=torch.int32, device=q.device)
         _hip.check(lib.aa_stage2_select(qb.data_ptr(), abar.data_ptr(), *_hip.t3(k), mask.data_ptr(), coords.data_ptr(),
                                         counts.data_ptr(), B, H, k.shape[1], N, D, BS, STEP, sm, args.theta * v4.LOG2E,
-                                        _hip.AA_GEOMETRY_AS_RUN, torch.cuda.current_stream().cuda_stream))
+                                        _hip.AA_GEOMETRY_AS_RUN, _hip.AA_DTYPE_BF16, torch.cuda.current_stream().cuda_stream))
         return coords, counts
 
     c0, n0 = select(qbar)

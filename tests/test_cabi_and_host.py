@@ -54,24 +54,27 @@ def test_error_codes_without_touching_the_gpu():
     buf = ctypes.create_string_buffer(4096 + 64)
     p = (ctypes.addressof(buf) + 63) & ~63
     s = (2048 * 128 * 2, 2048 * 128, 128)
-    dense = lambda q, nq, nkv, n, d, qs=s: lib.aa_dense_causal_fwd(q, *qs, p, *s, p, *s, p, *s, 1, nq, nkv, n, d, 0.1, None)
+    dense = lambda q, nq, nkv, n, d, qs=s: lib.aa_dense_causal_fwd(q, *qs, p, *s, p, *s, p, *s, 1, nq, nkv, n, d, 0.1, 0, None)
     assert dense(None, 2, 2, 2048, 128) == 1 and b"q is NULL" in lib.aa_last_error()
     assert dense(p, 3, 2, 2048, 128) == 1 and b"divide" in lib.aa_last_error()
     assert dense(p, 2, 2, 2048, 64) == 2 and b"head_dim" in lib.aa_last_error()
     assert dense(p, 2, 2, 2000, 128) == 2
     assert dense(p + 2, 2, 2, 2048, 128) == 3 and b"aligned" in lib.aa_last_error()
     assert dense(p, 2, 2, 2048, 128, qs=(s[0], s[1], 132)) == 3
-    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1024, None, 1, 2, 2, 2048, 128, 128, 16, 0.1, 12.0, 0, 0, None)
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1024, None, 1, 2, 2, 2048, 128, 128, 16, 0.1, 12.0, 0, 0, 0, None)
     assert rc == 1 and b"workspace" in lib.aa_last_error()
-    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, 0, None)
+    rc = lib.aa_anchor_attn_fwd(p, *s, p, *s, p, *s, p, *s, p, 1 << 40, None, 1, 2, 2, 2048 + 128, 128, 128, 16, 0.1, 12.0, 0, 0, 1, None)
     assert rc == 2 and b"multiple" in lib.aa_last_error()
     big = (s[0], s[1], 16384)  # 2^20 rows x 32 KiB per row does not fit 32-bit byte offsets
-    rc = lib.aa_stage1_anchor_fwd(p, *big, p, *s, p, *s, p, p, p, 1, 2, 2, 1 << 20, 128, 128, 16, 0.1, 0, None)
+    rc = lib.aa_stage1_anchor_fwd(p, *big, p, *s, p, *s, p, p, p, 1, 2, 2, 1 << 20, 128, 128, 16, 0.1, 0, 0, None)
     assert rc == 2 and b"32-bit" in lib.aa_last_error()
-    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 8, 0.1, 0, None)
+    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 8, 0.1, 0, 0, None)
     assert rc == 2 and b"step" in lib.aa_last_error()
-    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 7, None)
+    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 7, 0, None)
     assert rc == 1 and b"scale_mode" in lib.aa_last_error()
+    rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 0, 5, None)
+    assert rc == 1 and b"dtype" in lib.aa_last_error()
+    assert lib.aa_version() == 2
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -61,7 +61,7 @@ def _packed_lists(hip, coords, counts, N, step=STEP, bs=BS):
     return out, counts
 
 
-def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP, bs=BS):
+def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP, bs=BS, dtype="bf16"):
     """Sets equal except excused keys (flip distance < BAND); returns number of excused keys."""
     S = bs * step
     B, Hq = got_counts.shape[:2]
@@ -79,11 +79,11 @@ def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused,
                 if sym.size == 0:
                     continue
                 if qbar is None:
-                    qbar = ao.pooled_queries(Q[b, h], bs)
-                    abar, mean = ao.pooled_anchors(M[b, h], bs)
+                    qbar = ao.pooled_queries(Q[b, h], bs, dtype)
+                    abar, mean = ao.pooled_anchors(M[b, h], bs, dtype)
                 rows = slice(bb * step, (bb + 1) * step)
                 for j in sym:
-                    d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta)
+                    d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta, dtype)
                     assert d < BAND, f"key {j} (b={b},h={h},bb={bb}) differs and is {d:.4g} from any decision flip"
                     excused += 1
     assert excused <= max_excused, f"{excused} near-threshold disagreements"
@@ -179,7 +179,8 @@ def test_stage3_matches_oracle_given_same_state(mods, llama_small):
 def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP, bs=BS):
     hip, v4, st, ao = mods
     Q, K, V = _np(q, k, v)
-    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta)
+    dtype = "fp16" if q.dtype == torch.float16 else "bf16"
+    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta, dtype=dtype)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     out, ratio = v4.anchor_attn(qd, kd, vd, block_size=bs, step=step, difference=theta)
     B, H, N, _ = q.shape
@@ -188,7 +189,8 @@ def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP, bs=BS):
     np.testing.assert_allclose(M.cpu().numpy(), res.M, atol=3e-4)
     coords, counts = st.select_stripes_packed(qd, kd, M, bs, step, theta * LOG2E, B, H, N, D, SM)
     got, got_counts = _packed_lists(hip, coords, counts, N, step, bs)
-    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step, bs)
+    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step, bs, dtype)
+    assert out.dtype == q.dtype
     err = np.abs(out.float().cpu().numpy() - res.out)
     assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
     want_ratio = got_counts.sum() / ((B * H * N * N / (bs * step)) // 2)
@@ -282,6 +284,62 @@ def test_other_block_sizes(mods, bs, step, n_bb, hq, hkv, theta, seed):
     q, k, v, _ = _case(n_bb * bs * step, hq, hkv, max(8, n_bb * bs * step // 100), seed=seed)
     res, _ = _end_to_end(mods, q, k, v, theta, max_excused=8, step=step, bs=bs)
     assert res.counts.sum() > 0 and res.counts[:, :, 0].sum() == 0
+
+
+# ------------------------------------------------------------------------------------ fp16 tensors
+@pytest.mark.parametrize("n_bb,hq,hkv,bs,step,theta,seed,base", [
+    (3, 8, 2, 128, 16, 12.0, 401, 5e5),    # Llama grouping
+    (4, 7, 1, 128, 16, 12.0, 402, 1e6),    # Qwen grouping, RoPE base 1e6
+    (5, 4, 2, 64, 16, 13.0, 403, 5e5),     # another block size
+    (2, 2, 1, 128, 32, 11.0, 404, 5e5),    # step 32
+])
+def test_fp16_tensors_end_to_end(mods, n_bb, hq, hkv, bs, step, theta, seed, base):
+    """The reference's kernels also take fp16 tensors (every .to(dtype) then rounds to fp16: scaled queries,
+    probabilities, pooled queries and anchors, stage-2 scores, output).  Same checks as for bf16, against the oracle
+    in fp16 mode: anchors, index sets, outputs, ratio."""
+    q, k, v, _ = _case(n_bb * bs * step, hq, hkv, 32 * n_bb, seed=seed, rope_base=base, dtype=torch.float16)
+    res, out = _end_to_end(mods, q, k, v, theta, max_excused=8, step=step, bs=bs)
+    assert res.counts.sum() > 0 and out.dtype == torch.float16
+
+
+def test_fp16_stages_and_dense_baseline(mods):
+    """fp16: stage 1 against the oracle, pooling bit-exact (also the pooling fused into stage 1: one-call == staged),
+    stage 3 given the same state, the dense baseline against float64 library attention, and no mixing of types."""
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(3 * S, 4, 2, 96, seed=411, dtype=torch.float16)
+    Q, K, V = _np(q, k, v)
+    res = ao.anchor_attn_reference(Q, K, V, difference=12.0, dtype="fp16")
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
+    np.testing.assert_allclose(M.cpu().numpy(), res.M, atol=3e-4)
+    np.testing.assert_allclose(L.cpu().numpy(), res.L, rtol=5e-4)
+    err = np.abs(st.acc_rows(Acc).cpu().numpy() / L.cpu().numpy()[..., None] - res.Acc / res.L[..., None])
+    assert err.max() < 2e-3 and err.mean() < 1e-4
+    qbar, abar = st.pool_q_anchor(qd, torch.from_numpy(res.M).cuda(), BS)
+    assert qbar.dtype == torch.float16 and abar.dtype == torch.float16
+    for h in range(H):
+        assert np.array_equal(qbar[0, h].float().cpu().numpy(), ao.pooled_queries(Q[0, h], BS, "fp16"))
+        assert np.array_equal(abar[0, h].float().cpu().numpy(), ao.pooled_anchors(res.M[0, h], BS, "fp16")[0])
+    fused, ratio = v4.anchor_attn(qd, kd, vd, difference=12.0)
+    staged, ratio2 = v4.anchor_attn_without_anchor(qd, kd, vd, difference=12.0)
+    assert torch.equal(fused, staged) and float(ratio) == float(ratio2)
+    coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM)
+    out = v4._stage3(qd, kd, vd, coords, counts, L, M, Acc, SM, BS, STEP)
+    lists, cnts = _packed_lists(hip, coords, counts, N)
+    want = ao.stage3_sparse(Q, K, V, lists, cnts, M.cpu().numpy(), L.cpu().numpy(), st.acc_rows(Acc).cpu().numpy(), SM, dtype="fp16")
+    err = np.abs(out.float().cpu().numpy() - want)
+    assert err.max() <= 4e-3 and err.mean() <= 3e-4          # fp16 output: eight times finer than bf16
+    # the bf16 run of the same values differs (other rounding points), so the type switch is live
+    ob = v4.anchor_attn(qd.bfloat16(), kd.bfloat16(), vd.bfloat16(), return_computational_ratio=False)
+    assert ob.dtype == torch.bfloat16 and not torch.equal(ob.float(), fused.float())
+    dense = v4.dense_causal_attention(qd, kd, vd)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    e = (dense.cpu().double() - ref).abs()
+    assert dense.dtype == torch.float16 and e.max() < 4e-3 and e.mean() < 2e-4
+    with pytest.raises(AssertionError):
+        v4.anchor_attn(qd, kd.bfloat16(), vd.bfloat16())
 
 
 def test_theta_minus_inf_two_big_blocks_equals_library_attention(mods):
@@ -399,7 +457,7 @@ def test_entry_assertions_and_error_codes(mods):
     with pytest.raises(AssertionError):
         v4.anchor_attn(q[:, :, :1536], q[:, :, :1536], q[:, :, :1536], block_size=48, step=16)  # not one of 16 ... 256
     lib = hip.lib()
-    rc = lib.aa_dense_causal_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 2, 2048, 128, 0.1, None)
+    rc = lib.aa_dense_causal_fwd(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 2, 2048, 128, 0.1, 0, None)
     assert rc == 1 and b"NULL" in lib.aa_last_error()
 
 
@@ -447,7 +505,7 @@ def test_intended_geometry_mode(mods):
     # (looser than the oracle bound: the stage-1 bf16 scale chain is part of the operator, not of plain attention)
     assert e.max() < 4e-2 and e.mean() < 2e-3
     lib = hip.lib()
-    assert lib.aa_stage2_select(1, 1, 1, 0, 0, 128, 1, 1, 1, 1, 2, 2, 2048, 128, 128, 16, 0.1, 1.0, 5, None) == 1
+    assert lib.aa_stage2_select(1, 1, 1, 0, 0, 128, 1, 1, 1, 1, 2, 2, 2048, 128, 128, 16, 0.1, 1.0, 5, 0, None) == 1
     assert b"geometry" in lib.aa_last_error()
 
 
@@ -718,6 +776,22 @@ def test_triton_promotion_rule_live(mods, tmp_path):
     for i in range(8):
         assert np.array_equal(ao.pooled_anchors(r["pool_m"][i], 128)[0], r["pool_abar"][i])
     assert np.abs(ours - exact).max() <= np.abs(r["pool_qbar"] - exact).max() <= 0.02
+    # ---- the same on fp16 tensors: the chains, the stage-2 test and the anchor pooling run in fp16
+    hx = r["h_x"]
+    for name in ("d128", "d64", "odd"):
+        sm = float(r[f"sm_{name}"])
+        assert np.array_equal(r[f"h_constexpr_{name}"], ao.q1_scale_chain(hx, sm, mode="bf16_chain", dtype="fp16"))
+        assert np.array_equal(r[f"h_runtime_{name}"], ao.q3_scale_chain(hx, sm, dtype="fp16"))
+    # stage-2 score in fp16: the multiply and the cast compile into one instruction that rounds the exact product once
+    sc, _ = ao.stage2_scores(r["h_s2_dot"][:, None], np.ones((1, 1), np.float32), float(r["s2_sm"]), "fp16")
+    assert np.array_equal(sc[:, 0], r["h_s2_qk"])
+    hit = (sc[:, 0] + np.float32(float(r["s2_theta"]) * ao.LOG2E)) >= r["h_s2_anchor"]
+    assert np.array_equal(hit, r["h_s2_hit"].astype(bool))
+    for i in range(8):
+        assert np.array_equal(ao.pooled_anchors(r["pool_m"][i], 128, "fp16")[0], r["h_pool_abar"][i])
+    exact = r["h_pool_q"].reshape(8, 16, 128, 128).astype(np.float64).mean(axis=2)
+    ours = np.stack([ao.pooled_queries(r["h_pool_q"][i], 128, "fp16") for i in range(8)])
+    assert np.abs(ours - exact).max() <= np.abs(r["h_pool_qbar"] - exact).max() <= 0.01
 
 
 def test_pooling_precision_reading_is_immaterial(mods):

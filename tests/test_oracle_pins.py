@@ -252,18 +252,17 @@ def test_stage3_multiplicity_closed_form(small):
     assert (sel & wmask).any()
 
 
-@pytest.mark.parametrize("bs,step,n_bb", [(16, 16, 5), (32, 32, 3), (64, 16, 4), (256, 16, 2)])
-def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
-    """block_size is a parameter of all three stages (pooling width, candidate range [bs, bb*S - bs), big block
-    S = bs*step, window [0,S) U [bb*S, r]).  Independent route for every block size the reference's assert admits:
-    float64 window/selection masks and the multiplicity closed form for the output, torch bf16 casts and float64 dots
-    for the selection - none of it shares code with the oracle's tile loops."""
+def _closed_form_check(bs, step, n_bb, dtype):
+    """The whole operator against an independent route: float64 window/selection masks and the multiplicity closed form
+    for the output, torch casts to the 16-bit type and float64 dots for the selection - none of it shares code with the
+    oracle's tile loops."""
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float16
     S_ = bs * step
     N = n_bb * S_
-    q, k, v, _ = make_qkv(N, 2, 1, n_stripes=max(8, N // 64), seed=300 + bs)
+    q, k, v, _ = make_qkv(N, 2, 1, n_stripes=max(8, N // 64), seed=300 + bs, dtype=tdt)
     Q, K, V = _np(q, k, v)
     theta = 12.0
-    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta)
+    res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta, dtype=dtype)
     assert res.counts[:, :, 0].sum() == 0 and res.counts.sum() > 0
     r = np.arange(N)[:, None]
     j = np.arange(N)[None, :]
@@ -274,12 +273,12 @@ def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
     for h in range(2):
         # ---- selection, independently
         qt = torch.from_numpy(Q[0, h])
-        qbar = (qt.view(N // bs, bs, D).double().sum(1) / bs).float().to(torch.bfloat16)
-        s1 = ao.q1_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        qbar = (qt.view(N // bs, bs, D).double().sum(1) / bs).float().to(tdt)
+        s1 = ao.q1_scale_chain(Q[0, h], SM, dtype=dtype).astype(np.float64) @ k64.T
         m_rows = np.where(wmask, s1, -np.inf).max(1)                       # the anchors are the windowed row maxima
         np.testing.assert_allclose(res.M[0, h], m_rows, atol=2e-4)
-        abar = (torch.from_numpy(res.M[0, h]).view(N // bs, bs).double().sum(1) / bs).float().to(torch.bfloat16)
-        sc = ((qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (SM * ao.LOG2E)).float().to(torch.bfloat16)
+        abar = (torch.from_numpy(res.M[0, h]).view(N // bs, bs).double().sum(1) / bs).float().to(tdt)
+        sc = ((qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (SM * ao.LOG2E)).float().to(tdt)
         hit = ((sc.float() + diff) >= abar.float()[:, None]).view(n_bb, step, N).any(1)
         sel = np.zeros((N, N), bool)
         for bb in range(n_bb):
@@ -290,13 +289,61 @@ def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
             assert len(set(want.tolist()) ^ set(got.tolist())) <= 2          # float64 vs float32 dots at a boundary
             sel[bb * S_:(bb + 1) * S_, got] = True
         # ---- output: multiplicity closed form
-        s3 = ao.q3_scale_chain(Q[0, h], SM).astype(np.float64) @ k64.T
+        s3 = ao.q3_scale_chain(Q[0, h], SM, dtype=dtype).astype(np.float64) @ k64.T
         a = np.where(wmask, s1, -np.inf)
         b = np.where(sel, s3, -np.inf)
         mx = np.maximum(a.max(1), b.max(1))
         w = np.exp2(a - mx[:, None]) + np.exp2(b - mx[:, None])
         err = np.abs(res.out[0, h] - (w @ v64) / w.sum(1)[:, None])
         assert err.max() < 2e-2 and err.mean() < 1.5e-3
+    return res
+
+
+@pytest.mark.parametrize("bs,step,n_bb", [(16, 16, 5), (32, 32, 3), (64, 16, 4), (256, 16, 2)])
+def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
+    """block_size is a parameter of all three stages (pooling width, candidate range [bs, bb*S - bs), big block
+    S = bs*step, window [0,S) U [bb*S, r]): every block size the reference's assert admits."""
+    _closed_form_check(bs, step, n_bb, "bf16")
+
+
+# ---------------------------------------------------------------- fp16 tensors
+def test_fp16_rounding_matches_torch_cast():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(200000, generator=g) * torch.logspace(-9, 5, 200000)
+    ties = torch.arange(1, 2049, dtype=torch.float32) * 2.0 ** -11 + 1.0          # 1 + k/2048: every second one is a tie
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1e-8, -3e-8, 65504.0, 65519.9, 65520.0, 1e6, 6.1e-5, 5.9e-8])
+    for t in (x, ties, special):
+        want = t.to(torch.float16).float().numpy()
+        got = ao.rnd16(t.numpy(), "fp16")
+        assert np.array_equal(want.view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(ao.rnd16(x.numpy(), "bf16"), ao.rn16(x.numpy()))
+    with pytest.raises(ValueError):
+        ao.rnd16(x.numpy(), "fp8")
+
+
+def test_fp16_scale_chains_are_torch_half_arithmetic():
+    """With fp16 tensors the stage-1 chain rounds both constants and both products to fp16 (torch evaluates a
+    half*half product as a float32 product rounded once), the stage-3 chain rounds once."""
+    q = torch.randn(4096, D, generator=torch.Generator().manual_seed(2)).to(torch.float16)
+    t1 = (q * torch.tensor(SM, dtype=torch.float16)) * torch.tensor(ao.LOG2E, dtype=torch.float16)
+    assert t1.dtype == torch.float16
+    assert np.array_equal(t1.float().numpy(), ao.q1_scale_chain(q.float().numpy(), SM, dtype="fp16"))
+    t3 = ((q.float() * torch.tensor(SM, dtype=torch.float32)) * torch.tensor(ao.LOG2E, dtype=torch.float32)).to(torch.float16)
+    assert np.array_equal(t3.float().numpy(), ao.q3_scale_chain(q.float().numpy(), SM, dtype="fp16"))
+    # fp16 keeps three more bits than bf16: the chain stays within 1e-3 of the exact scale (bf16: 1.0017)
+    r = ao.q1_scale_chain(np.full(1, 64.0, np.float32), SM, dtype="fp16")[0] / (64.0 * SM * ao.LOG2E)
+    assert abs(r - 1.0) < 1e-3 and (ao.q1_scale_chain(q.float().numpy(), SM, dtype="fp16") != ao.q1_scale_chain(q.float().numpy(), SM)).any()
+
+
+@pytest.mark.parametrize("bs,step,n_bb", [(128, 16, 3), (64, 16, 4)])
+def test_fp16_operator_by_independent_closed_form(bs, step, n_bb):
+    res = _closed_form_check(bs, step, n_bb, "fp16")
+    # the decision-boundary helper works in fp16 steps too
+    b = ao.stage2_decision_boundary(24.5, 12.0, "fp16")
+    for eps, want in ((+1e-4, True), (-1e-4, False)):
+        sc = ao.rnd16(np.array([b + eps], np.float32), "fp16")[0]
+        assert bool(np.float32(sc + np.float32(12.0 * ao.LOG2E)) >= np.float32(24.5)) is want
+    assert res.counts.sum() > 0
 
 
 def test_stage3_constant_values_give_that_value(small):
@@ -408,3 +455,35 @@ def test_scale_chains_match_triton_compiled_outputs():
         xb = ao.stage2_decision_boundary(float(anchor[i]), theta)
         if float(raw[i]) != xb:  # (exactly on the midpoint the bf16 tie rule decides)
             assert (float(raw[i]) > xb) == bool(fx["s2_hit"][i])
+
+
+def test_fp16_chains_match_triton_compiled_outputs():
+    """The fp16 half of the same probe (tests/golden/triton_scale_chain_probe_fp16.npz): on fp16 tensors the constexpr
+    form keeps both products in fp16, the run-time form rounds once; the stage-2 score is one rounding of the exact
+    product (the multiply and the cast compile into one mixed-precision instruction)."""
+    import os
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "triton_scale_chain_probe_fp16.npz"))
+    unbits = lambda b: b.view(np.float16).astype(np.float32)
+    x = unbits(fx["x_f16_bits"])
+    assert x.size > 4000
+    for name in ("d128", "d64", "odd"):
+        sm = float(fx[f"sm_{name}"])
+        want1, want3 = unbits(fx[f"constexpr_{name}_f16_bits"]), unbits(fx[f"runtime_{name}_f16_bits"])
+        assert np.array_equal(ao.q1_scale_chain(x, sm, mode="bf16_chain", dtype="fp16"), want1)
+        assert np.array_equal(ao.q3_scale_chain(x, sm, dtype="fp16"), want3)
+        assert (want1 != want3).sum() > 500
+        assert (want1 != ao.q1_scale_chain(x, sm, mode="bf16_chain", dtype="bf16")).sum() > 500  # and not the bf16 chain
+    dot, anchor, qk = fx["s2_dot"], unbits(fx["s2_anchor_f16_bits"]), unbits(fx["s2_qk_f16_bits"])
+    sm, theta = float(fx["s2_sm"]), float(fx["s2_theta"])
+    # the compiled stage-2 score: one rounding of the exact product (the oracle's fp16 reading), which differs from the
+    # two roundings of the source text on exact ties only
+    sc, raw = ao.stage2_scores(dot[:, None].astype(np.float32), np.ones((1, 1), np.float32), sm, "fp16")  # dot * 1 = dot
+    sc, raw = sc[:, 0], raw[:, 0]
+    assert np.array_equal(sc, qk)
+    two = ao.rnd16(raw, "fp16")
+    odd = np.nonzero(two != qk)[0]
+    assert 0 < odd.size <= 8
+    for i in odd:
+        assert abs(float(raw[i]) - float(two[i])) == abs(float(raw[i]) - float(qk[i]))  # exact ties only
+    hit = (sc + np.float32(theta * ao.LOG2E)) >= anchor
+    assert np.array_equal(hit, fx["s2_hit"].astype(bool)) and 0.2 < hit.mean() < 0.8

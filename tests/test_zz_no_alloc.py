@@ -32,12 +32,12 @@ def _select_both_ways(n_ctx, hq, hkv, n_stripes, seed, theta):
     coords_a, counts_a = outputs()
     mask = torch.empty((lib.aa_mask_words(B, H, N, BS, STEP),), dtype=torch.int32, device="cuda")
     _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(k), mask.data_ptr(), coords_a.data_ptr(),
-                                    counts_a.data_ptr(), B, H, hkv, N, D, BS, STEP, SM, theta * LOG2E, 0, stream))
+                                    counts_a.data_ptr(), B, H, hkv, N, D, BS, STEP, SM, theta * LOG2E, 0, _hip.AA_DTYPE_BF16, stream))
     coords_b, counts_b = outputs()
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats()["allocation.all.allocated"]
     _hip.check(lib.aa_stage2_select_static(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(k), coords_b.data_ptr(),
-                                           counts_b.data_ptr(), B, H, hkv, N, D, BS, STEP, SM, theta * LOG2E, 0, stream))
+                                           counts_b.data_ptr(), B, H, hkv, N, D, BS, STEP, SM, theta * LOG2E, 0, _hip.AA_DTYPE_BF16, stream))
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats()["allocation.all.allocated"] == before  # nothing came from torch's allocator either
     return coords_a, counts_a, coords_b, counts_b
@@ -59,7 +59,7 @@ def test_static_scratch_entry_point_equals_the_allocating_one_twice_in_a_row():
     # a problem beyond the static capacity is refused before anything is launched
     need = lib.aa_mask_words(1, 64, 131072, BS, STEP) * 4
     assert need > _hip.AA_STATIC_SCRATCH_BYTES
-    rc = lib.aa_stage2_select_static(1, 1, 1, 0, 0, 128, 1, 1, 1, 64, 8, 131072, D, BS, STEP, SM, 17.0, 0, None)
+    rc = lib.aa_stage2_select_static(1, 1, 1, 0, 0, 128, 1, 1, 1, 64, 8, 131072, D, BS, STEP, SM, 17.0, 0, 0, None)
     assert rc == 2 and b"static scratch" in lib.aa_last_error()
     # the headline layer shape fits
     assert lib.aa_mask_words(1, 32, 131072, BS, STEP) * 4 <= _hip.AA_STATIC_SCRATCH_BYTES

@@ -6,7 +6,8 @@ The reference's stage-1 kernel takes ``sm_scale`` as ``tl.constexpr`` and evalua
 evaluates the same expression with ``sm_scale`` as a run-time float argument (anchor_attn_v4.py:9,66).  This script
 runs both forms on every finite bf16 value, and the element-wise part of the stage-2 selection test
 (get_mask_test.py:86,96-101) on 65536 near-threshold cases, and the pooling lines (get_mask_test.py:75-84) on
-eight big blocks, and writes the results to an ``.npz``:
+eight big blocks - each once for bf16 tensors and once for fp16 tensors (keys prefixed ``h_``) - and writes the
+results to an ``.npz``:
 
     python tests/triton_promotion_probe.py OUT.npz [cpu|cuda]
 
@@ -68,12 +69,12 @@ def _pool(q_ptr, m_ptr, qbar_ptr, abar_ptr, step: tl.constexpr, BLOCK_SZ: tl.con
     tl.store(abar_ptr + tl.arange(0, step)[:, None] + tl.arange(0, 1)[None, :], anchors.to(tl.float32))
 
 
-def stage2_cases(device, sm_scale, theta):
-    """65536 (dot, anchor) pairs whose scaled score lies within a few bf16 steps of the decision boundary."""
+def stage2_cases(device, sm_scale, theta, dtype=torch.bfloat16):
+    """65536 (dot, anchor) pairs whose scaled score lies within a few steps of the 16-bit type of the decision boundary."""
     g = torch.Generator().manual_seed(4)
-    anchors = (torch.rand(4096, generator=g) * 38 + 2).to(torch.bfloat16)
+    anchors = (torch.rand(4096, generator=g) * 38 + 2).to(dtype)
     target = anchors.float() - theta * 1.44269504                       # scaled score at the boundary
-    step = torch.clamp(target.abs(), min=1e-3) * 2.0 ** -8               # about one bf16 step there
+    step = torch.clamp(target.abs(), min=1e-3) * (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11)  # about one step there
     delta = torch.linspace(-2.5, 2.5, 16)[None, :] * step[:, None]
     dot = ((target[:, None] + delta) / (sm_scale * 1.44269504)).float().reshape(-1)
     return dot.to(device), anchors[:, None].expand(4096, 16).reshape(-1).contiguous().to(device)
@@ -86,6 +87,13 @@ def all_finite_bf16(device):
     pad = (-x.numel()) % 256
     x = torch.cat([x, torch.zeros(pad)])
     return x.to(torch.bfloat16).to(device)
+
+
+def all_finite_fp16(device):
+    x = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    x = x[torch.isfinite(x)]
+    pad = (-x.numel()) % 256
+    return torch.cat([x, torch.zeros(pad, dtype=torch.float16)]).to(device)
 
 
 def main(out_path, device):
@@ -116,6 +124,30 @@ def main(out_path, device):
     for i in range(8):
         _pool[(1,)](pq[i], pm[i], qbar[i], abar[i], 16, 128, 128, tl.bfloat16)
     res.update(pool_q=pq.float().cpu().numpy(), pool_m=pm.cpu().numpy(), pool_qbar=qbar.cpu().numpy(), pool_abar=abar.cpu().numpy())
+    # ---- the same three probes on fp16 tensors (keys prefixed h_): the reference selects dtype = tl.float16 for them
+    hx = all_finite_fp16(device)
+    res["h_x"] = hx.float().cpu().numpy()
+    for name, sm in (("d128", 128 ** -0.5), ("d64", 0.125), ("odd", 0.1)):
+        a = torch.empty(hx.numel(), dtype=torch.float32, device=device)
+        b = torch.empty_like(a)
+        grid = (hx.numel() // 256,)
+        _scale_constexpr[grid](hx, a, sm, 256)
+        _scale_runtime[grid](hx, b, sm, 256)
+        res[f"h_constexpr_{name}"] = a.cpu().numpy()
+        res[f"h_runtime_{name}"] = b.cpu().numpy()
+    sm, theta = 128 ** -0.5, 12.0
+    dot, anchors = stage2_cases(device, sm, theta, torch.float16)
+    qk = torch.empty(dot.numel(), dtype=torch.float32, device=device)
+    hit = torch.empty(dot.numel(), dtype=torch.int32, device=device)
+    _stage2_decision[(dot.numel() // 256,)](dot, anchors, qk, hit, theta * 1.44269504, sm, tl.float16, 256)
+    res.update(h_s2_dot=dot.cpu().numpy(), h_s2_anchor=anchors.float().cpu().numpy(), h_s2_qk=qk.cpu().numpy(),
+               h_s2_hit=hit.cpu().numpy().astype(np.uint8))
+    hq = pq.to(torch.float16)
+    hqbar = torch.empty_like(qbar)
+    habar = torch.empty_like(abar)
+    for i in range(8):
+        _pool[(1,)](hq[i], pm[i], hqbar[i], habar[i], 16, 128, 128, tl.float16)
+    res.update(h_pool_q=hq.float().cpu().numpy(), h_pool_qbar=hqbar.cpu().numpy(), h_pool_abar=habar.cpu().numpy())
     np.savez_compressed(out_path, **res)
 
 
