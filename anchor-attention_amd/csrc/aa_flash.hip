@@ -144,14 +144,35 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const int group = p.n_q_heads / p.n_kv_heads;
   const int nq = MODE == kSparse ? p.q_blocks_per_wg : 1;
   const int n_qunit = p.n_ctx / (BM * nq);
-  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qunit, group);
-  const int g = vid % group;  vid /= group;
-  int qunit = vid % n_qunit;  vid /= n_qunit;
-  const int kvh = vid % p.n_kv_heads;
-  const int b = vid / p.n_kv_heads;
-  const int hq = kvh * group + g;
-  qunit = n_qunit - 1 - qunit;  // longest rows first (later big blocks also carry the longest index lists)
   const int S = p.big_block;
+  int g, qunit, kvh, b;
+  const uint32_t n_pairs = (uint32_t)(p.batch * p.n_kv_heads) * (uint32_t)(p.n_ctx / S);
+  if (MODE == kSparse && n_pairs % 8u == 0u) {
+    // Stage 3's work per (KV head, big block) pair is the length of the pair's index lists, which depends on the data:
+    // a head whose queries select many keys would keep its XCD busy long after the others have finished if whole
+    // heads were tied to XCDs.  So the unit that stays on one XCD (and shares its L2) is the pair - the query blocks of
+    // a big block and the heads of a KV group gather the same rows - and consecutive pairs, ordered latest big block
+    // first, go round-robin over the XCDs with a rotation, so that every XCD sees every head and every depth.
+    const uint32_t per_pair = (uint32_t)group * (uint32_t)(S / (BM * nq));  // work-groups of a pair
+    const uint32_t n_units = (uint32_t)(p.batch * p.n_kv_heads);
+    const uint32_t xcd = blockIdx.x % 8u, k = blockIdx.x / 8u;
+    const uint32_t kp = k / per_pair, within = k % per_pair;
+    const uint32_t pair = kp * 8u + (xcd + kp) % 8u;
+    const int bb_ = p.n_ctx / S - 1 - (int)(pair / n_units);
+    const uint32_t unit = pair % n_units;
+    g = within % group;
+    qunit = bb_ * (S / (BM * nq)) + (int)(within / group);
+    kvh = unit % p.n_kv_heads;
+    b = unit / p.n_kv_heads;
+  } else {
+    uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qunit, group);
+    g = vid % group;  vid /= group;
+    qunit = vid % n_qunit;  vid /= n_qunit;
+    kvh = vid % p.n_kv_heads;
+    b = vid / p.n_kv_heads;
+    qunit = n_qunit - 1 - qunit;  // longest rows first (later big blocks also carry the longest index lists)
+  }
+  const int hq = kvh * group + g;
   const int bb = qunit * nq * BM / S;  // (all blocks of a work-group lie in one big block: the host picks q_blocks_per_wg so)
   const int64_t bh = (int64_t)b * p.n_q_heads + hq;
 
