@@ -7,11 +7,15 @@ on this package's own MFMA kernel - the baseline "built on the same kernels"), "
 patch.py:36-45,142-144); the competitor patterns of the reference are not part of this package and raise
 ``ValueError``.  In transformers 5 the attention product is selected by
 name through ``AttentionInterface``, so patching is: register the plug once, point the model's config at it,
-and copy the pattern's parameters onto the config (patch.py:106-109 does the same ``setattr`` loop).
+and copy the pattern's parameters onto the config (patch.py:106-109 does the same ``setattr`` loop).  Like the
+reference (patch.py:146-157), every pattern but "default" also makes the model return logits for the last position
+only and evaluates the MLPs in chunks of 32768 positions (``model_forward.py``).
 """
 import copy
 
 from my_utils import Logger
+
+from anchor_attn.src.modules.model_forward import MLP_CHUNK_TOKENS, chunk_mlp_over_tokens, keep_last_token_logits
 
 ATTENTION_CONFIG_EXAMPLE = {
     "default": {},
@@ -50,7 +54,9 @@ def patch_model(model, pattern: str, config: dict = None):
 
     pattern: "default" (leave as is), "flash" (the framework's library attention), "dense" (causal attention on this
              package's own kernel), "anchor_attn" or "anchor_attn_lite" (same operator, same defaults).
-    config : for the anchor patterns ``{"block_size_M": 128, "theta": 12, "step": 16}`` (the defaults).
+    config : for the anchor patterns ``{"block_size_M": 128, "theta": 12, "step": 16}`` (the defaults).  Two optional
+             keys steer the model-level patches the reference applies unconditionally: ``"last_token_logits"``
+             (default True) and ``"mlp_chunk_tokens"`` (default 32768; 0 leaves the MLPs alone).
     """
     from transformers import PreTrainedModel
     if not isinstance(model, PreTrainedModel):
@@ -64,6 +70,8 @@ def patch_model(model, pattern: str, config: dict = None):
         return model
     cfg = get_config_example(pattern)
     cfg.update(config or {})
+    last_token_logits = bool(cfg.pop("last_token_logits", True))
+    mlp_chunk_tokens = int(cfg.pop("mlp_chunk_tokens", MLP_CHUNK_TOKENS))
     if pattern == "flash":
         model.set_attn_implementation("sdpa")
     elif pattern == "dense":
@@ -74,5 +82,8 @@ def patch_model(model, pattern: str, config: dict = None):
         model.set_attn_implementation(_register()[0])
         for k, v in cfg.items():
             setattr(model.config, k, v)
+    if last_token_logits:
+        keep_last_token_logits(model)
+    chunk_mlp_over_tokens(model, mlp_chunk_tokens)
     Logger.log(f"replace attention with {pattern}: {cfg}")
     return model

@@ -42,6 +42,49 @@ def test_patch_model_validation_and_config():
     assert set(get_config_example()) == {"default", "flash", "dense", "anchor_attn", "anchor_attn_lite"}
 
 
+def test_model_level_patches_last_token_logits_and_chunked_mlp():
+    """Every pattern but "default" also patches the model as the reference does (patch.py:146-157): the forward
+    returns float32 logits of the last position only (causal_model_forward.py:124-125) and the MLPs run over chunks
+    of the sequence (llama_mlp_forward.py:46-58) - neither changes a value."""
+    from anchor_attn import patch_model
+    from anchor_attn.src.modules import model_forward
+    assert model_forward.MLP_CHUNK_TOKENS == 32768
+    ref = _tiny()
+    x = torch.randint(0, 1000, (2, 300))
+    with torch.no_grad():
+        full = ref(x).logits
+    for pattern in ("flash", "dense", "anchor_attn", "anchor_attn_lite"):
+        m = _tiny()
+        m.load_state_dict(ref.state_dict())
+        patch_model(m, pattern, {"mlp_chunk_tokens": 64})  # 300 positions = four full chunks and a ragged one
+        assert all(layer.mlp._mlp_chunk_tokens == 64 for layer in m.model.layers)
+        with torch.no_grad():
+            last = m(x).logits
+            assert last.shape == (2, 1, 1000) and last.dtype == torch.float32
+            assert torch.allclose(last, full[:, -1:], atol=1e-5)
+            # a caller that names the positions it wants, or passes labels, gets them
+            assert torch.allclose(m(x, logits_to_keep=0).logits, full, atol=1e-5)
+            assert m(x, logits_to_keep=7).logits.shape == (2, 7, 1000)
+            with_loss = m(x, labels=x)
+            assert with_loss.logits.shape == (2, 300, 1000)
+            assert abs(float(with_loss.loss) - float(ref(x, labels=x).loss)) < 1e-5
+            # the chunked MLP is the MLP
+            h = torch.randn(2, 300, 512)
+            assert torch.allclose(m.model.layers[0].mlp(h), ref.model.layers[0].mlp(h), atol=1e-6)
+        # patching again wraps nothing twice and only moves the chunk size
+        fwd, mlp_fwd = m.forward, m.model.layers[0].mlp.forward
+        patch_model(m, pattern)
+        assert m.forward is fwd and m.model.layers[0].mlp.forward is mlp_fwd
+        assert m.model.layers[0].mlp._mlp_chunk_tokens == 32768
+    # both can be declined
+    m = _tiny()
+    m.load_state_dict(ref.state_dict())
+    patch_model(m, "anchor_attn", {"last_token_logits": False, "mlp_chunk_tokens": 0})
+    with torch.no_grad():
+        assert m(x).logits.shape == (2, 300, 1000)
+    assert not hasattr(m.config, "last_token_logits") and not hasattr(m.config, "mlp_chunk_tokens")
+
+
 def test_dense_pattern_on_cpu_is_plain_attention():
     """Without a GPU the dense plug has only its framework branch; a model patched with it computes what the
     unpatched model computes (prefill and cached decode)."""
@@ -52,7 +95,7 @@ def test_dense_pattern_on_cpu_is_plain_attention():
     patch_model(m, "dense")
     x = torch.randint(0, 1000, (1, 200))
     with torch.no_grad():
-        assert torch.allclose(ref(x).logits, m(x).logits, atol=1e-5)
+        assert torch.allclose(ref(x).logits, m(x, logits_to_keep=0).logits, atol=1e-5)
         assert torch.equal(ref.generate(x, max_new_tokens=3, do_sample=False), m.generate(x, max_new_tokens=3, do_sample=False))
 
 
@@ -67,7 +110,7 @@ def test_short_prefill_and_decode_take_the_dense_branch():
     x = torch.randint(0, 1000, (2, 300))
     with torch.no_grad():
         a = ref(x).logits
-        b = m(x).logits
+        b = m(x, logits_to_keep=0).logits
         assert torch.allclose(a, b, atol=1e-5)
         ga = ref.generate(x, max_new_tokens=4, do_sample=False)
         gb = m.generate(x, max_new_tokens=4, do_sample=False)
