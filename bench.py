@@ -148,8 +148,10 @@ def gemm_reference(dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=10,
+                    help="untimed calls before the timed ones (the first ~10 calls on an idle GPU run up to 25 %% slower "
+                         "while its clocks ramp up)")
     ap.add_argument("--workload", default="config2_llama8b_128k", choices=sorted(WORKLOADS))
     ap.add_argument("--theta", type=float, default=12.0)
     ap.add_argument("--qbar-mode", default="shared", choices=["shared", "literal"])
