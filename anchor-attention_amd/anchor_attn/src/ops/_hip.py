@@ -62,13 +62,23 @@ def lib() -> ctypes.CDLL:
                 f"{path} is missing: build it with `make -C anchor-attention_amd/csrc` "
                 "(there is no fallback implementation)"
             )
-        handle = ctypes.CDLL(path)
-        for name, (res, args) in _SIGNATURES.items():
-            fn = getattr(handle, name)
-            fn.restype = res
-            fn.argtypes = args
+        handle = bind(path)
+        version = handle.aa_version()
+        if version >= 1000:
+            raise AnchorAttnHipError(f"{path} is a timing-only build (aa_version() = {version}) that leaves part of a "
+                                     "kernel out; it computes wrong results and is not loaded as the operator")
         _lib = handle
     return _lib
+
+
+def bind(path: str) -> ctypes.CDLL:
+    """Open a build of the library and declare the C signatures on it (no check of what kind of build it is)."""
+    handle = ctypes.CDLL(path)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(handle, name)
+        fn.restype = res
+        fn.argtypes = args
+    return handle
 
 
 def check(rc: int) -> None:

@@ -48,6 +48,17 @@ constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (
 
 enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
 
+// Timing-only ablations.  A build with -DAA_ABLATE=n (`make ablations`) leaves out one ingredient of the kernel so
+// that its cost can be measured (bench_ablations.py); such a build computes WRONG results on purpose, reports
+// aa_version() >= 1000 and is refused by the Python loader.  0, the default, is the product.
+//   1  exp2 of the soft-max replaced by a pass-through        4  (sparse) no tile loop: state in, output out
+//   2  no soft-max arithmetic at all (mask, max, exp, sum)    5  (sparse) accumulator state not loaded
+//   3  no K/V tile loads inside the tile loop                 6  (sparse) at most two tiles per query block
+//                                                             7  (sparse) 4 and 5 together
+#ifndef AA_ABLATE
+#define AA_ABLATE 0
+#endif
+
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -211,10 +222,14 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   } else if (MODE == kDense) {
     n_tiles = (R0 + BM) / kBN;
   } else {
-    cnt = p.counts[bh * (p.n_ctx / S) + bb];
     cap = max(bb * S - 2 * p.block_size, 0);  // capacity of the big block's list (a multiple of 4)
+    // (counts and indices come from device memory the caller filled: a count beyond the capacity or an index beyond
+    // the context is clamped rather than followed out of bounds)
+    cnt = max(0, min(p.counts[bh * (p.n_ctx / S) + bb], cap));
     cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
     n_tiles = (cnt + kBN - 1) / kBN;
+    if (AA_ABLATE == 4 || AA_ABLATE == 7) n_tiles = 0;
+    if (AA_ABLATE == 6) n_tiles = min(n_tiles, 2);
   }
   // first key (anchor, dense) or first list position (sparse) of tile i
 #define AA_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
@@ -230,6 +245,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     if (pos + 1 >= cnt) v.y = 0;
     if (pos + 2 >= cnt) v.z = 0;
     if (pos + 3 >= cnt) v.w = 0;
+    const uint32_t last = (uint32_t)p.n_ctx - 1u;
+    v.x = (int)min((uint32_t)v.x, last);
+    v.y = (int)min((uint32_t)v.y, last);
+    v.z = (int)min((uint32_t)v.z, last);
+    v.w = (int)min((uint32_t)v.w, last);
     *reinterpret_cast<int4*>(&sm.idx[4 * tid]) = v;
   };
   // (uniform over the work-group; not conditioned on the count, see above.  Later blocks of the work-group find the
@@ -268,7 +288,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        const floatx4 t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256));
+        floatx4 t = {0.f, 0.f, 0.f, 0.f};
+        if (AA_ABLATE != 5 && AA_ABLATE != 7) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256));
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
       }
@@ -355,12 +376,13 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     t0 = fmaxf(t0, t3);                                                              \
     mx = max_with_other_half(t0);                                                     \
   }
+#define AA_EXP2(x) ((AA_ABLATE == 1 || AA_ABLATE == 2) ? (x) : fast_exp2(x))
   // p = exp2(s) for accumulator registers 4c .. 4c+3 of one half, summed and rounded into the P^T fragment words
 #define AA_EXP_CHUNK(sx, pw, sum, c)                                                 \
   {                                                                                  \
-    const float e0 = fast_exp2(sx[4 * (c) + 0]), e1 = fast_exp2(sx[4 * (c) + 1]);    \
-    const float e2 = fast_exp2(sx[4 * (c) + 2]), e3 = fast_exp2(sx[4 * (c) + 3]);    \
-    sum += e0; sum += e1; sum += e2; sum += e3;                                      \
+    const float e0 = AA_EXP2(sx[4 * (c) + 0]), e1 = AA_EXP2(sx[4 * (c) + 1]);        \
+    const float e2 = AA_EXP2(sx[4 * (c) + 2]), e3 = AA_EXP2(sx[4 * (c) + 3]);        \
+    if (AA_ABLATE != 2) { sum += e0; sum += e1; sum += e2; sum += e3; }              \
     pw[(c) >> 1][2 * ((c) & 1) + 0] = T::pack(e0, e1);                                 \
     pw[(c) >> 1][2 * ((c) & 1) + 1] = T::pack(e2, e3);                                 \
   }
@@ -442,7 +464,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       for (int n = 0; n < 8; ++n) {
         AA_OPERAND_FETCH(n + kDist)
         AA_S_MFMA(s0, n);
-        AA_FETCH_ONE(n)
+        if (AA_ABLATE != 3) { AA_FETCH_ONE(n) }
         AA_FENCE;
       }
 
@@ -453,8 +475,12 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         AA_S_MFMA(s1, n);
         AA_FENCE;
       }
-      AA_MASK(s0, 0)
-      AA_ROWMAX(s0, mx0)
+      if (AA_ABLATE != 2) {
+        AA_MASK(s0, 0)
+        AA_ROWMAX(s0, mx0)
+      } else {
+        mx0 = -INFINITY;
+      }
       const bool moved0 = __any(m_ref + mx0 > m_run);
       if (moved0) {
         // slow path: some row's max grew.  Lanes whose max did not move get shift 0 and alpha 1 (exact).
@@ -501,8 +527,12 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s1[r] -= shift0;
       }
-      AA_MASK(s1, 1)
-      AA_ROWMAX(s1, mx1)
+      if (AA_ABLATE != 2) {
+        AA_MASK(s1, 1)
+        AA_ROWMAX(s1, mx1)
+      } else {
+        mx1 = -INFINITY;
+      }
       const bool moved1 = __any(m_ref + mx1 > m_run);
       if (moved1) {
         // as above, except that O^T is rescaled only after the P0 V0 products in flight have been added

@@ -56,6 +56,8 @@ extern "C" {
 #define AA_GEOMETRY_AS_RUN 0
 #define AA_GEOMETRY_INTENDED 1
 
+/* 2 for this ABI.  1000 + n marks a timing-only build (`make ablations`, AA_ABLATE = n) that leaves part of a kernel out and
+ * computes wrong results on purpose; such a build is for bench_ablations.py only and the Python loader refuses it. */
 int aa_version(void);
 const char* aa_last_error(void);
 
@@ -138,7 +140,10 @@ int aa_stage2_select_static(const void* qbar, const void* abar,
 /* ---- stage 3: fine-grained sparse flash attention ------------------------------------------
  * Replaces _triton_stripe_sparse_attn_fwd_kernel_step3 (anchor_attn_v4.py:7-105; launch
  * :246-268): resumes the online softmax from (M, L, acc_frag) over the K/V rows gathered at the
- * big block's selected indices and writes out = round16(acc / l).  M, L, acc_frag are read-only. */
+ * big block's selected indices and writes out = round16(acc / l).  M, L, acc_frag are read-only.
+ * coords and counts are read as they are found in device memory: a count below 0 or above the list's capacity is
+ * clamped to it and an index outside [0, n_ctx) to the nearest valid row, so stale or corrupt lists give wrong
+ * values but no access outside the tensors. */
 int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                          const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
                          const void* v, int64_t v_sb, int64_t v_sh, int64_t v_sn,

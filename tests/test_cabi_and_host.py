@@ -190,3 +190,22 @@ def test_recall_bookkeeping_on_cpu():
     assert RECALL_THRESHOLDS == (0.01, 0.005)
     assert row == {"sparsity_ratio": 0.25, "recall@0.01": 0.7, "recall@0.005": 0.4}
     assert record_recall_ratios(out, out, 0.5, thresholds=(1e-6,)) == {"sparsity_ratio": 0.5, "recall@1e-06": 1.0}
+
+
+def test_timing_only_builds_are_refused_as_the_operator(monkeypatch):
+    """`make ablations` builds variants of the library that leave part of a kernel out; they report
+    aa_version() >= 1000 and the loader does not accept them in place of the product build."""
+    import glob
+    import os
+
+    from anchor_attn.src.ops import _hip
+    libs = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "..", "anchor-attention_amd", "csrc", "_ablations", "*.so")))
+    if not libs:
+        pytest.skip("timing-only builds not present (make -C anchor-attention_amd/csrc ablations)")
+    for path in libs:
+        handle = _hip.bind(path)
+        assert handle.aa_version() >= 1001
+    monkeypatch.setenv("ANCHOR_ATTN_HIP_LIB", libs[0])
+    monkeypatch.setattr(_hip, "_lib", None)
+    with pytest.raises(_hip.AnchorAttnHipError, match="timing-only"):
+        _hip.lib()

@@ -461,6 +461,30 @@ def test_entry_assertions_and_error_codes(mods):
     assert rc == 1 and b"NULL" in lib.aa_last_error()
 
 
+def test_stage3_clamps_counts_and_indices_it_is_given(mods):
+    """The index lists and counts are device memory that the caller hands to stage 3.  Counts beyond a list's capacity
+    and indices outside the context are clamped by the kernel instead of being followed: the call returns, the output
+    is finite, and rows of the first big block (whose list has no capacity) are exactly the stage-1 result."""
+    hip, v4, st, ao = mods
+    q, k, v, _ = _case(4 * S, 4, 2, 64, seed=91)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    B, H, N, _ = q.shape
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM)
+    good = v4._stage3(qd, kd, vd, coords, counts, L, M, Acc, SM, BS, STEP)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    bad_coords = torch.randint(-2 ** 31, 2 ** 31 - 1, coords.shape, generator=g, device="cuda", dtype=torch.int64).to(torch.int32)
+    bad_counts = torch.full_like(counts, 2 ** 30)
+    bad_counts[:, 0::2] = -7
+    out = v4._stage3(qd, kd, vd, bad_coords, bad_counts, L, M, Acc, SM, BS, STEP)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out[:, :, :S], good[:, :, :S])
+    # negative counts are empty lists: those heads come out as they do with counts of zero
+    empty = v4._stage3(qd, kd, vd, coords, torch.zeros_like(counts), L, M, Acc, SM, BS, STEP)
+    assert torch.equal(out[:, 0::2], empty[:, 0::2])
+
+
 # ------------------------------------------------------------------------------------ larger sizes
 def test_constant_values_at_32k(mods):
     """Size-independent property at the 32k shape: if every V row is the same vector, every output
