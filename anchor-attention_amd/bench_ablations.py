@@ -26,10 +26,10 @@ sys.path.insert(0, os.path.dirname(HERE))
 STAGE1 = {1: "exp2 of the soft-max replaced by a pass-through",
           2: "no soft-max arithmetic (mask, max, exp, sum); scores converted as they are",
           3: "no K/V tile loads inside the tile loop"}
-STAGE3 = {4: "no tile loop: statistics and accumulator state in, output out",
+STAGE3 = {4: "no tile loop: statistics and accumulator state in, output out (the unused query loads are compiled away)",
           5: "accumulator state not loaded (tile loop kept)",
           6: "at most two tiles per query block",
-          7: "no tile loop and no accumulator state: queries in, output out",
+          7: "no tile loop and no accumulator state: only the output is written (the unused query loads are compiled away)",
           1: "exp2 of the soft-max replaced by a pass-through",
           2: "no soft-max arithmetic",
           3: "no K/V tile loads inside the tile loop"}
