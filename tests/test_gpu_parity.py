@@ -559,7 +559,7 @@ def test_theta_sweep_tooling(mods):
     assert wide[1]["recall@0.01"] >= wide[0]["recall@0.01"]
 
 
-def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples):
+def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16"):
     """Stages 1 and 3 on sampled (head, row) pairs, recomputed in float64 on the host (P rounded to bf16 as the
     kernels do) from the kernel's own index lists; returns the per-row max errors."""
     N = q.shape[2]
@@ -572,23 +572,23 @@ def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples):
         K1 = k[0, kv, keys1].double().cpu().numpy()
         V1 = v[0, kv, keys1].double().cpu().numpy()
         qrow = q[0, h, r].float().cpu().numpy()
-        q1 = ao.q1_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        q1 = ao.q1_scale_chain(qrow[None], SM, dtype=dtype)[0].astype(np.float64)
         s1 = K1 @ q1
         m1 = s1.max()
         p1 = np.exp2(s1 - m1)
         l1 = p1.sum()
-        a1 = ao.rn16(p1.astype(np.float32)).astype(np.float64) @ V1
+        a1 = ao.rnd16(p1.astype(np.float32), dtype).astype(np.float64) @ V1
         assert abs(float(M[0, h, r]) - m1) < 3e-4
         assert abs(float(L[0, h, r]) - l1) / l1 < 1e-3
         lst = index_list(h, bb)
-        q3 = ao.q3_scale_chain(qrow[None], SM)[0].astype(np.float64)
+        q3 = ao.q3_scale_chain(qrow[None], SM, dtype=dtype)[0].astype(np.float64)
         if lst.size:
             K3 = k[0, kv, lst].double().cpu().numpy()
             V3 = v[0, kv, lst].double().cpu().numpy()
             s3 = K3 @ q3
             m = max(m1, s3.max())
             p3 = np.exp2(s3 - m)
-            num = a1 * np.exp2(m1 - m) + ao.rn16(p3.astype(np.float32)).astype(np.float64) @ V3
+            num = a1 * np.exp2(m1 - m) + ao.rnd16(p3.astype(np.float32), dtype).astype(np.float64) @ V3
             den = l1 * np.exp2(m1 - m) + p3.sum()
         else:
             num, den = a1, l1
@@ -598,7 +598,7 @@ def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples):
     return errs
 
 
-def _full_size_sampled_parity(mods, workload, theta, seed, pairs, samples, ratio_range, max_flips_per_pair=3):
+def _full_size_sampled_parity(mods, workload, theta, seed, pairs, samples, ratio_range, max_flips_per_pair=3, dtype="bf16"):
     """One BASELINE workload at its stated size through all three stages: staged entry points == one-call entry
     point bit for bit; stage 2 of the sampled (head, big block) pairs against the oracle's stage-2 arithmetic
     (identical index sets except keys within the flip band); sampled output rows against a float64 host
@@ -606,6 +606,8 @@ def _full_size_sampled_parity(mods, workload, theta, seed, pairs, samples, ratio
     hip, v4, st, ao = mods
     from bench import make_inputs
     q, k, v = make_inputs(workload, seed, "shared", "cuda:0")
+    if dtype == "fp16":
+        q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
     B, H, N, _ = q.shape
     group = H // k.shape[1]
     n_bb = N // S
@@ -633,22 +635,22 @@ def _full_size_sampled_parity(mods, workload, theta, seed, pairs, samples, ratio
         Qb = q[0, h, rows].float().cpu().numpy()
         Mb = M[0, h, rows].cpu().numpy()
         Kc = k[0, h // group, BS:bb * S - BS].float().cpu().numpy()
-        qbar = ao.pooled_queries(Qb, BS)
-        abar, mean = ao.pooled_anchors(Mb, BS)
-        sc, _ = ao.stage2_scores(qbar, Kc, SM)
+        qbar = ao.pooled_queries(Qb, BS, dtype)
+        abar, mean = ao.pooled_anchors(Mb, BS, dtype)
+        sc, _ = ao.stage2_scores(qbar, Kc, SM, dtype)
         want = (np.nonzero(((sc + np.float32(theta * LOG2E)) >= abar[:, None]).any(axis=0))[0] + BS).astype(np.int32)
         got = index_list(h, bb)
         assert np.all(np.diff(got) > 0)
         assert got.size == 0 or (got[0] >= BS and got[-1] < bb * S - BS)
         diff = np.setxor1d(got, want)
         for j in diff:
-            d_ = ao.stage2_flip_distance(qbar, abar, mean, k[0, h // group, int(j)].float().cpu().numpy(), SM, theta)
+            d_ = ao.stage2_flip_distance(qbar, abar, mean, k[0, h // group, int(j)].float().cpu().numpy(), SM, theta, dtype)
             assert d_ < BAND, (workload, theta, h, bb, int(j), d_)
         assert diff.size <= max_flips_per_pair, (workload, theta, h, bb, diff.size)
         excused += diff.size
     # ---- stages 1 and 3 on sampled rows
     samples = [(h % H, r % N) for h, r in samples]
-    errs = _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples)
+    errs = _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype)
     assert len(errs) == len(samples)
     return cnt, excused
 
@@ -662,6 +664,17 @@ def test_full_size_128k_sampled_parity(mods):
         pairs=[(0, -1), (13, 17), (31, 1), (22, 40)],
         samples=[(0, 0), (0, N - 1), (5, 2047), (9, 2048), (17, 70000), (31, N - 2048), (26, int(rng.integers(S, N)))],
         ratio_range=(0.001, 0.05))
+
+
+def test_full_size_128k_fp16_tensors(mods):
+    """The headline shape with fp16 tensors (the reference takes the element type from its inputs): same checks, with
+    the oracle's fp16 roundings - among them the single rounding of stage 2's scaled score."""
+    N = 131072
+    _full_size_sampled_parity(
+        mods, "config2_llama8b_128k", 12.0, 4,
+        pairs=[(1, -1), (14, 20), (30, 3)],
+        samples=[(0, N - 1), (6, 2048), (19, 81234), (31, N - 2047)],
+        ratio_range=(0.001, 0.05), dtype="fp16")
 
 
 @pytest.mark.parametrize("theta", [10.0, 14.0])
