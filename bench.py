@@ -156,6 +156,7 @@ def main():
     ap.add_argument("--theta", type=float, default=12.0)
     ap.add_argument("--qbar-mode", default="shared", choices=["shared", "literal"])
     ap.add_argument("--seed", type=int, default=2024)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"], help="element type of q, k, v and the output")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm-ref", action="store_true",
                     help="skip the library bf16 GEMM that is timed after the run as the practical MFMA rate of this box")
@@ -177,6 +178,8 @@ def main():
     D, BS, STEP, S = 128, 128, 16, 2048
     sm = 1.0 / math.sqrt(D)
     q, k, v = make_inputs(args.workload, args.seed, args.qbar_mode, dev)
+    if args.dtype == "fp16":
+        q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
     out = torch.empty_like(q)
     if args.calibrate_copy:
         src = torch.ones(2**28, dtype=torch.float32, device=dev)
@@ -213,7 +216,7 @@ def main():
             counts = torch.empty((1, hq, n_ctx // S, 1), dtype=torch.int32, device=dev)
         _hip.check(lib.aa_stage2_select(qbar.data_ptr(), abar.data_ptr(), *_hip.t3(k), mask.data_ptr(), coords.data_ptr(),
                                         counts.data_ptr(), 1, hq, hkv, n_ctx, D, BS, STEP, sm, theta2, _hip.AA_GEOMETRY_AS_RUN,
-                                        _hip.AA_DTYPE_BF16, torch.cuda.current_stream().cuda_stream))
+                                        _hip.dtype_code(q), torch.cuda.current_stream().cuda_stream))
         ev[i][3].record()
         v4._stage3(q, k, v, coords, counts, L, M, Acc, sm, BS, STEP, out=out)
         ev[i][4].record()
@@ -256,7 +259,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {"workload": args.workload, "n_ctx": n_ctx, "n_q_heads": hq, "n_kv_heads": hkv, "head_dim": D,
                    "theta": args.theta, "block_size": BS, "step": STEP, "qbar_mode": args.qbar_mode, "seed": args.seed},
