@@ -185,33 +185,47 @@ def test_patched_model_equals_dense_model_when_the_window_covers_everything():
 
 @pytest.mark.gpu
 def test_patched_qwen2_model(monkeypatch):
-    """The same plug under Qwen2 (attention biases, its own config class): window-covers-everything equality with
-    the dense model, and a real sparse prefill that stays finite and reports a ratio."""
+    """The same plug under Qwen2 (attention biases, its own config class, optional sliding-window layers):
+    window-covers-everything equality with the dense model, and a real sparse prefill that stays finite and reports a
+    ratio.  A sliding-window layer arrives with a mask that is not purely causal and takes the plug's dense branch."""
     from transformers import Qwen2Config, Qwen2ForCausalLM
 
     from anchor_attn import patch_model
-    from anchor_attn.src.modules.qwen2 import anchor_attention as plug
-    torch.manual_seed(0)
-    cfg = Qwen2Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
-                      num_key_value_heads=2, vocab_size=1000, max_position_embeddings=16384, rope_theta=1e6)
-    assert cfg.hidden_size // cfg.num_attention_heads == 128
-    ref = Qwen2ForCausalLM(cfg).eval().to(torch.bfloat16).cuda()
-    m = Qwen2ForCausalLM(cfg).eval().to(torch.bfloat16).cuda()
-    m.load_state_dict(ref.state_dict())
-    patch_model(m, "anchor_attn", {"theta": -1e4})
-    x = torch.randint(0, 1000, (1, 2 * 2048 + 5), device="cuda")
-    with torch.no_grad():
-        a = ref(x, logits_to_keep=32).logits.float()
-        b = m(x, logits_to_keep=32).logits.float()
-    assert torch.isfinite(b).all() and (a - b).abs().max() < 0.08 * a.abs().max()
+    import anchor_attn.src.modules.llama.anchor_attention as plug
+
+    def config(**kw):  # a model keeps the config object it is given: one per model, or patching one patches both
+        return Qwen2Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                           num_key_value_heads=2, vocab_size=1000, max_position_embeddings=16384, rope_theta=1e6, **kw)
+
+    assert config().hidden_size // config().num_attention_heads == 128
+    for kw in ({}, {"use_sliding_window": True, "sliding_window": 1024, "max_window_layers": 1}):
+        torch.manual_seed(0)
+        ref = Qwen2ForCausalLM(config(**kw)).eval().to(torch.bfloat16).cuda()
+        m = Qwen2ForCausalLM(config(**kw)).eval().to(torch.bfloat16).cuda()
+        assert m.config is not ref.config
+        m.load_state_dict(ref.state_dict())
+        patch_model(m, "anchor_attn", {"theta": -1e4})
+        assert ref.config._attn_implementation != plug.ATTN_NAME and m.config._attn_implementation == plug.ATTN_NAME
+        if kw:
+            assert m.config.layer_types == ["full_attention", "sliding_attention"]
+        masks = []
+        inner = plug._dense
+        monkeypatch.setattr(plug, "_dense", lambda q, k, v, mask, *a: (masks.append(mask is not None), inner(q, k, v, mask, *a))[1])
+        x = torch.randint(0, 1000, (1, 2 * 2048 + 5), device="cuda")
+        with torch.no_grad():
+            a = ref(x, logits_to_keep=32).logits.float()
+            b = m(x, logits_to_keep=32).logits.float()
+        assert torch.isfinite(b).all() and (a - b).abs().max() < 0.08 * a.abs().max()
+        # full-attention layers: the operator plus a dense tail without a mask; the sliding layer: dense with its mask
+        assert masks == ([False, True] if kw else [False, False]), masks
+        monkeypatch.setattr(plug, "_dense", inner)
     patch_model(m, "anchor_attn", {"theta": 12})
-    import anchor_attn.src.modules.llama.anchor_attention as llama_plug
-    monkeypatch.setattr(llama_plug, "record_ratio", True)
+    monkeypatch.setattr(plug, "record_ratio", True)
     y = torch.randint(0, 1000, (1, 3 * 2048), device="cuda")
     with torch.no_grad():
         c = m(y, logits_to_keep=1).logits
-    assert torch.isfinite(c).all() and plug.anchor_attention_forward is llama_plug.anchor_attention_forward
-    assert 0 < float(llama_plug.last_ratio) <= 1.0
+    assert torch.isfinite(c).all()
+    assert 0 < float(plug.last_ratio) <= 1.0
 
 
 @pytest.mark.gpu
