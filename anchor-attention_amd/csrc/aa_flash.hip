@@ -55,6 +55,7 @@ enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
 //   2  no soft-max arithmetic at all (mask, max, exp, sum)    5  (sparse) accumulator state not loaded
 //   3  no K/V tile loads inside the tile loop                 6  (sparse) at most two tiles per query block
 //                                                             7  (sparse) 4 and 5 together
+//   8  no work-group barrier at the end of a tile             9  neither the barrier nor the wait for the tile's loads
 #ifndef AA_ABLATE
 #define AA_ABLATE 0
 #endif
@@ -588,8 +589,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
     for (int m = 0; m < 4; ++m) v_rd[m] += buf_step;
     buf_step = -buf_step;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
-    __syncthreads();
+    if (AA_ABLATE != 9) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
+    if (AA_ABLATE != 8 && AA_ABLATE != 9) __syncthreads();
   }
 #undef AA_TILE_KEY0
 #undef AA_KEY_OF
