@@ -209,3 +209,21 @@ def test_timing_only_builds_are_refused_as_the_operator(monkeypatch):
     monkeypatch.setattr(_hip, "_lib", None)
     with pytest.raises(_hip.AnchorAttnHipError, match="timing-only"):
         _hip.lib()
+
+
+def test_bench_cli_contract_without_a_gpu():
+    """bench.py measures one GPU: a request for more exits with a message that says so (before anything touches a
+    device); the FLOP model it reports is the documented closed form."""
+    import subprocess
+    import sys
+    root = os.path.join(os.path.dirname(__file__), "..")
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+    sys.path.insert(0, root)
+    import bench
+    f1, f2, f3 = bench.flops(32, 131072, 855140)
+    assert f1 == 32 * (136 + 63 * 392) * 4 * 128 * 128 * 128            # 6.67 TFLOP of window tiles
+    assert f2 == 32 * 2 * 16 * 128 * sum(bb * 2048 - 256 for bb in range(1, 64))
+    assert f3 == 4 * 128 * 2048 * 855140
+    assert abs((f1 + f2 + f3) / 1e12 - 8.10) < 0.01
+    assert set(bench.WORKLOADS) == {"config0_llama8b_4k", "config1_llama8b_32k", "config2_llama8b_128k", "config3_qwen7b_64k"}
