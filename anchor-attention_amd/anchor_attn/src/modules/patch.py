@@ -12,6 +12,7 @@ reference (patch.py:146-157), every pattern but "default" also makes the model r
 only and evaluates the MLPs in chunks of 32768 positions (``model_forward.py``).
 """
 import copy
+import json
 
 from my_utils import Logger
 
@@ -49,14 +50,30 @@ def _register():
     return ATTN_NAME, DENSE_ATTN_NAME
 
 
-def patch_model(model, pattern: str, config: dict = None):
+def _config_dict(config):
+    """``config`` as the reference's callers pass it: None, a dict, or the JSON text of one (test_hf.py hands its
+    ``--config`` string straight through; patch.py:62-74 parses it and reports bad JSON as ``ValueError``)."""
+    if config is None:
+        return {}
+    if isinstance(config, str):
+        try:
+            config = json.loads(config)
+        except json.JSONDecodeError as e:
+            raise ValueError(f"Configuration string is not valid JSON: {e}")
+    if not isinstance(config, dict):
+        raise ValueError(f"config must be a dict or the JSON text of one, got {type(config).__name__}")
+    return config
+
+
+def patch_model(model, pattern: str, config=None):
     """Patch ``model`` (a transformers ``PreTrainedModel`` of the Llama or Qwen2 family) in place.
 
     pattern: "default" (leave as is), "flash" (the framework's library attention), "dense" (causal attention on this
              package's own kernel), "anchor_attn" or "anchor_attn_lite" (same operator, same defaults).
-    config : for the anchor patterns ``{"block_size_M": 128, "theta": 12, "step": 16}`` (the defaults).  Two optional
-             keys steer the model-level patches the reference applies unconditionally: ``"last_token_logits"``
-             (default True) and ``"mlp_chunk_tokens"`` (default 32768; 0 leaves the MLPs alone).
+    config : None, a dict or a JSON string; for the anchor patterns ``{"block_size_M": 128, "theta": 12, "step": 16}``
+             (the defaults; keys left out keep them).  Two optional keys with no counterpart in the reference steer
+             the model-level patches the reference applies unconditionally: ``"last_token_logits"`` (default True) and
+             ``"mlp_chunk_tokens"`` (default 32768; 0 leaves the MLPs alone).
     """
     from transformers import PreTrainedModel
     if not isinstance(model, PreTrainedModel):
@@ -69,7 +86,7 @@ def patch_model(model, pattern: str, config: dict = None):
     if pattern == "default":
         return model
     cfg = get_config_example(pattern)
-    cfg.update(config or {})
+    cfg.update(_config_dict(config))
     last_token_logits = bool(cfg.pop("last_token_logits", True))
     mlp_chunk_tokens = int(cfg.pop("mlp_chunk_tokens", MLP_CHUNK_TOKENS))
     if pattern == "flash":
