@@ -8,6 +8,10 @@ library attention (pattern "flash").
 There is no checkpoint or dataset involved: weights and tokens are synthetic, so the sparsity a trained
 model would show is not reproduced - the numbers are timings of the code path, and say so.
 
+Next to the bare forward, each pattern is also timed the way the reference's driver measures "prefill time"
+(test_hf.py:24-36): host wall-clock around ``model.generate(input_ids, attention_mask=ones, max_new_tokens=1,
+num_beams=1, do_sample=False)``, which includes building the KV cache and the generation loop's bookkeeping.
+
     python bench_model_prefill.py                       # config 4
     python bench_model_prefill.py --layers 2 --n-ctx 8192   # quick check
 """
@@ -77,6 +81,23 @@ def main():
                 best = (ms, attn, [float(r) for _, _, r in spans if r is not None], out)
         return best
 
+    def generate_one_token_ms(reps):
+        """The reference's prefill metric: wall-clock of generate(max_new_tokens=1) (its return is a host-side token
+        tensor, so the call ends synchronised, as in the reference)."""
+        ones = torch.ones_like(tokens)
+        best = None
+        for _ in range(reps + 1):
+            torch.cuda.synchronize()
+            t = time.time()
+            with torch.no_grad():
+                seq = model.generate(input_ids=tokens, attention_mask=ones, max_new_tokens=1, num_beams=1, do_sample=False,
+                                     pad_token_id=0)
+            int(seq[0, -1])  # the token is on the host: the prefill has finished
+            ms = (time.time() - t) * 1000.0
+            best = ms if best is None else min(best, ms)
+        assert seq.shape[1] == args.n_ctx + 1
+        return best
+
     patch_model(model, "anchor_attn", {"theta": args.theta})
     from transformers import AttentionInterface
     AttentionInterface.register(plug.ATTN_NAME, timed_plug(plug.anchor_attention_forward))
@@ -85,9 +106,11 @@ def main():
     res = {"workload": f"llama3.1-8b architecture, {args.layers} layers, random-init bf16, N={args.n_ctx}, theta={args.theta}",
            "prefill_ms_anchor_attn": ms, "attention_ms": attn_ms, "attention_share": attn_ms / ms,
            "mean_sparsity_ratio": sum(ratios) / max(len(ratios), 1), "logits_finite": bool(torch.isfinite(logits).all())}
+    res["generate_1_token_ms_anchor_attn"] = generate_one_token_ms(1)
     if not args.no_dense:
         patch_model(model, "dense")
         dms, dattn, _, dlogits = prefill(1)
+        res["generate_1_token_ms_dense_own_kernel"] = generate_one_token_ms(1)
         res["prefill_ms_dense_own_kernel"] = dms
         res["attention_ms_dense_own_kernel"] = dattn
         res["speedup_vs_dense_own_kernel"] = dms / ms
