@@ -1,6 +1,6 @@
 """What each ingredient of the stage-1 and stage-3 kernels costs: timing-only builds against the product build.
 
-`make -C anchor-attention_amd/csrc ablations` builds nine variants of the library that each leave one thing out
+`make -C anchor-attention_amd/csrc ablations` builds ten variants of the library that each leave one thing out
 (AA_ABLATE in csrc/aa_flash.hip).  Their results are wrong on purpose, so they are never loaded as the operator;
 this script opens them next to the product build, gives every build the SAME inputs - queries, keys, values, and
 for stage 3 the statistics, accumulator state and index lists computed by the product build - and times one entry
@@ -27,7 +27,8 @@ STAGE1 = {1: "exp2 of the soft-max replaced by a pass-through",
           2: "no soft-max arithmetic (mask, max, exp, sum); scores converted as they are",
           3: "no K/V tile loads inside the tile loop",
           8: "no work-group barrier at the end of a tile",
-          9: "neither the barrier nor the wait for the tile's loads at the end of a tile"}
+          9: "neither the barrier nor the wait for the tile's loads at the end of a tile",
+          10: "nothing: the soft-max runs in full, but P.V takes a loop-invariant operand (dependency scores -> P -> P.V cut)"}
 STAGE3 = {4: "no tile loop: statistics and accumulator state in, output out (the unused query loads are compiled away)",
           5: "accumulator state not loaded (tile loop kept)",
           6: "at most two tiles per query block",
@@ -36,7 +37,8 @@ STAGE3 = {4: "no tile loop: statistics and accumulator state in, output out (the
           2: "no soft-max arithmetic",
           3: "no K/V tile loads inside the tile loop",
           8: "no work-group barrier at the end of a tile",
-          9: "neither the barrier nor the wait for the tile's loads at the end of a tile"}
+          9: "neither the barrier nor the wait for the tile's loads at the end of a tile",
+          10: "nothing: the soft-max runs in full, but P.V takes a loop-invariant operand (dependency cut)"}
 
 
 def main():

@@ -34,6 +34,8 @@
 //   K row r, chunk c  ->  slot c ^ (r & 15)          (row-per-lane 16-byte reads)
 //   V row r, chunk c  ->  slot c ^ ((r & 7) << 1)    (transposing 8-byte reads)
 // Both choices measure conflict-free for their read pattern (and each is 2-way conflicted for the other's).
+#include <type_traits>
+
 #include "aa_common.h"
 #include "aa_kernels.h"
 
@@ -56,6 +58,8 @@ enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
 //   3  no K/V tile loads inside the tile loop                 6  (sparse) at most two tiles per query block
 //                                                             7  (sparse) 4 and 5 together
 //   8  no work-group barrier at the end of a tile             9  neither the barrier nor the wait for the tile's loads
+//  10  the soft-max is computed in full (same instructions, same energy) but the second product takes a loop-invariant
+//      operand instead of P: the dependency scores -> soft-max -> P.V inside a wave is cut, nothing else changes
 #ifndef AA_ABLATE
 #define AA_ABLATE 0
 #endif
@@ -120,7 +124,7 @@ template <int MODE>
 __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, const char* vb, const uint32_t k_row_bytes,
                                                const uint32_t v_row_bytes, const uint32_t k_col, const uint32_t v_col, const int key0,
                                                const int tid, const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v,
-                                               const uint32_t (&k_voff)[4], const uint32_t (&v_voff)[4]) {
+                                               const uint32_t k_voff, const uint32_t v_voff) {
   const int j = n >> 1;  // load n: K (even n) or V (odd n) rows 16*j + ...
   if (MODE == kSparse) {
     const int row = (tid >> 4) + 16 * j;
@@ -128,10 +132,10 @@ __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, cons
     if ((n & 1) == 0) load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
     else load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
   } else {
-    // consecutive keys: the tile's first row goes into the (scalar) base address, the thread's row and chunk
-    // inside the tile are loop-invariant vector offsets - no vector arithmetic per tile
-    if ((n & 1) == 0) load16_to_lds(kb + (uint64_t)(uint32_t)key0 * k_row_bytes, k_voff[j], lds_k + 16 * j * kRowBytes);
-    else load16_to_lds(vb + (uint64_t)(uint32_t)key0 * v_row_bytes, v_voff[j], lds_v + 16 * j * kRowBytes);
+    // consecutive keys: the first row of the tile's j-th block of 16 rows goes into the (scalar) base address, the
+    // thread's row inside the block and its chunk are one loop-invariant vector offset - no vector arithmetic per tile
+    if ((n & 1) == 0) load16_to_lds(kb + (uint64_t)(uint32_t)(key0 + 16 * j) * k_row_bytes, k_voff, lds_k + 16 * j * kRowBytes);
+    else load16_to_lds(vb + (uint64_t)(uint32_t)(key0 + 16 * j) * v_row_bytes, v_voff, lds_v + 16 * j * kRowBytes);
   }
 }
 
@@ -264,12 +268,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const uint32_t k_col = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15)) * 16u;
   const uint32_t v_col = (uint32_t)((tid & 15) ^ (((tid >> 4) & 7) << 1)) * 16u;
   const uint32_t lds_k0 = lds_addr(sm.t.k[0]) + wave * 4 * kRowBytes, lds_v0 = lds_addr(sm.t.v[0]) + wave * 4 * kRowBytes;
-  uint32_t k_voff[4], v_voff[4];  // byte offset of this thread's chunk of tile row (tid >> 4) + 16*j from the tile's first row
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    k_voff[j] = ((tid >> 4) + 16 * j) * k_row_bytes + k_col;
-    v_voff[j] = ((tid >> 4) + 16 * j) * v_row_bytes + v_col;
-  }
+  // byte offset of this thread's chunk of row (tid >> 4) of a block of 16 tile rows from the block's first row
+  const uint32_t k_voff = (tid >> 4) * k_row_bytes + k_col, v_voff = (tid >> 4) * v_row_bytes + v_col;
   // (anchor mode with pooling) the work-group's raw query rows, fetched like a tile by the last tile's load slots
   const char* qblock = reinterpret_cast<const char*>(qp + (int64_t)R0 * p.q_sn);
   const uint32_t q_row_bytes = (uint32_t)p.q_sn * 2u;
@@ -388,7 +388,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     pw[(c) >> 1][2 * ((c) & 1) + 1] = T::pack(e2, e3);                                 \
   }
   // V operand fetch i (two transposing reads): i = (kb*2 + st)*4 + db
-#define AA_V_SRC(i) (v_rd[(i) & 3] + (uint32_t)((32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes))
+#define AA_V_SRC(i) (v_rd[(i) & 3] + (uint32_t)(rd_off + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes))
 #define AA_V_FETCH(i)                                                                                  \
   {                                                                                                    \
     vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(AA_V_SRC(i)));                     \
@@ -399,13 +399,19 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     typedef short shortx8 __attribute__((ext_vector_type(8)));                                         \
     const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);                \
     acc[(i) & 3] = T::mfma(*reinterpret_cast<const vec8*>(&av),                                        \
-                           *reinterpret_cast<const vec8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3]);         \
+                           AA_ABLATE == 10 ? qreg[(i) & 7] : *reinterpret_cast<const vec8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3]); \
   }
 #define AA_FENCE __builtin_amdgcn_sched_barrier(0)
 
-  int32_t buf_step = kTileBytes;  // what takes the read addresses to the other LDS buffer
-  for (int i = 0; i < n_tiles; ++i) {
-    const int buf = i & 1;
+  // One tile.  The LDS buffer it reads (BUF) is a compile-time constant - the loop below is unrolled by two - so that
+  // the buffer's offset is part of every LDS instruction's immediate offset and the read addresses are loop-invariant.
+  // Sparse mode, whose tile counts can be odd, keeps one copy of the tile (BUF = -1): the buffer is i & 1 and the read
+  // addresses step back and forth between the two buffers.
+  int32_t buf_step = kTileBytes;
+  auto run_tile = [&](auto buf_const, const int i) __attribute__((always_inline)) {
+    constexpr int kBuf = decltype(buf_const)::value;
+    constexpr uint32_t rd_off = kBuf > 0 ? kBuf * kTileBytes : 0;  // immediate part of the LDS read addresses
+    const int buf = kBuf >= 0 ? kBuf : (i & 1);
     const int key0 = AA_TILE_KEY0(i);
     if (MODE == kSparse && i + 1 < n_tiles && ((i + 1) & (kIdxWin / kBN - 1)) == 0) {
       // tile i+1 opens the next window; everyone finished reading the old one before the last barrier
@@ -422,13 +428,16 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     const int i_next = i + 1 < n_tiles ? i + 1 : i;
     const int key0_next = AA_TILE_KEY0(i_next);
     const bool fetch_queries = MODE == kAnchor && pool && i + 1 == n_tiles;  // wave-uniform
+    // (selects, not branches: the eight slots stay straight-line code; the base address is scalar, and the vector offset
+    // is chosen once per tile and operand kind)
+    const uint32_t k_voff_sel = fetch_queries ? q_voff : k_voff, v_voff_sel = fetch_queries ? q_voff : v_voff;
 #define AA_FETCH_ONE(n)                                                                                               \
-  if (MODE == kAnchor) { /* selects, not branches: the eight slots stay straight-line code */                        \
+  if (MODE == kAnchor) {                                                                                              \
     const int j_ = (n) >> 1;                                                                                          \
-    const char* kv_ = ((n) & 1) ? vbase + (uint64_t)(uint32_t)key0_next * v_row_bytes                                 \
-                                : kbase + (uint64_t)(uint32_t)key0_next * k_row_bytes;                                \
+    const char* kv_ = ((n) & 1) ? vbase + (uint64_t)(uint32_t)(key0_next + 16 * j_) * v_row_bytes                     \
+                                : kbase + (uint64_t)(uint32_t)(key0_next + 16 * j_) * k_row_bytes;                    \
     const char* q_ = qblock + (uint64_t)(64 * ((n) & 1) + 16 * j_) * q_row_bytes;                                     \
-    load16_to_lds(fetch_queries ? q_ : kv_, fetch_queries ? q_voff : (((n) & 1) ? v_voff[j_] : k_voff[j_]),           \
+    load16_to_lds(fetch_queries ? q_ : kv_, ((n) & 1) ? v_voff_sel : k_voff_sel,                                      \
                   (((n) & 1) ? lds_v0 : lds_k0) + (buf ^ 1) * kTileBytes + 16 * j_ * kRowBytes);                      \
   } else {                                                                                                            \
     tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,             \
@@ -442,7 +451,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       shortx4 vlo[16], vhi[16];  // V operand of slot 16 + i, i = (kb*2 + st)*4 + db
       u32x4 pw0[2], pw1[2];      // P^T fragments (bf16 pairs) of the two halves
       float mx0, mx1, sum0 = 0.f, sum1 = 0.f, shift0 = 0.f, alpha1 = 1.f;
-#define AA_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(32 * ((t) >> 3) * kRowBytes))
+#define AA_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(rd_off + 32 * ((t) >> 3) * kRowBytes))
 
       // The 32 MFMAs of a tile are slots 0..31 (16 for S^T, 16 for O^T); the operand of slot n is fetched from
       // LDS while slot n - kDist is issued.  The scheduling fences keep that distance: left alone, the reads sink
@@ -577,20 +586,33 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         AA_PV_MFMA(n - 16, pw1)
         AA_FENCE;
       }
+      if (AA_ABLATE == 10) {  // P is still formed: it only has to exist by the end of the tile
+        asm volatile("" ::"v"(pw0[0]), "v"(pw0[1]), "v"(pw1[0]), "v"(pw1[1]));
+      }
 #undef AA_OPERAND_FETCH
 #undef AA_S_MFMA
 #undef AA_K_FETCH
     }
 #undef AA_FETCH_ONE
 
-    // the read addresses follow the tiles into the other buffer
+    if (kBuf < 0) {  // the read addresses follow the tiles into the other buffer
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_rd[ks] += buf_step;
+      for (int ks = 0; ks < 8; ++ks) k_rd[ks] += buf_step;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) v_rd[m] += buf_step;
-    buf_step = -buf_step;
+      for (int m = 0; m < 4; ++m) v_rd[m] += buf_step;
+      buf_step = -buf_step;
+    }
     if (AA_ABLATE != 9) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
     if (AA_ABLATE != 8 && AA_ABLATE != 9) __syncthreads();
+  };
+  if (MODE == kSparse) {
+    for (int i = 0; i < n_tiles; ++i) run_tile(std::integral_constant<int, -1>{}, i);
+  } else {
+    // 128 query rows and 64-key tiles: the window of a query block always holds an even number of tiles
+    for (int i = 0; i < n_tiles; i += 2) {
+      run_tile(std::integral_constant<int, 0>{}, i);
+      run_tile(std::integral_constant<int, 1>{}, i + 1);
+    }
   }
 #undef AA_TILE_KEY0
 #undef AA_KEY_OF
