@@ -154,6 +154,11 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   constexpr int kTilesPerWg = WAVES / 2;         // two waves share one 128-key tile
   static_assert(kRowsPerWave % STEP == 0 && kItemsPerWave >= 1 && kRowsPerWave % 4 == 0, "a wave stages whole items");
   static_assert(ROWS % 64 == 0 && ROWS / 64 <= WAVES, "thresholds are staged 64 per wave");
+  // the swizzle is written with the row inside a wave's share on the load side (r & 15) and with the row inside a
+  // 32-row group on the read side (c32 & 15): the two agree only when a wave's share is whole groups of 16 rows; and
+  // the per-item mask words of a block live in lanes 0..63 of one register pair
+  static_assert(kRowsPerWave % 16 == 0, "a wave stages whole groups of 16 rows (the swizzle's period)");
+  static_assert(kBlockItems <= 64, "one lane per item of a block");
   __shared__ __attribute__((aligned(16))) char a_lds[2][ROWS * kSelRowBytes];
   __shared__ __attribute__((aligned(16))) float thr_lds[2][ROWS];
 

@@ -677,9 +677,10 @@ def test_full_size_128k_fp16_tensors(mods):
         ratio_range=(0.001, 0.05), dtype="fp16")
 
 
-@pytest.mark.parametrize("theta", [10.0, 14.0])
+@pytest.mark.parametrize("theta", [10.0, 11.0, 13.0, 14.0])
 def test_config2_theta_sweep_ends_at_128k(mods, theta):
-    """BASELINE config 2 at the two ends of its theta sweep.  theta = 14 admits ordinary keys next to the stripes:
+    """BASELINE config 2 over the rest of its theta sweep (the reference default +-2; theta = 12 is the headline test):
+    the two ends and the two points between.  theta = 14 admits ordinary keys next to the stripes:
     index lists are several times longer than at theta 12 (stage 3 refills its index window), and more keys sit
     close to the threshold."""
     N = 131072
