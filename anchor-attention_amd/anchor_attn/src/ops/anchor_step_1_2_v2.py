@@ -55,7 +55,7 @@ def acc_rows(Acc_frag: torch.Tensor) -> torch.Tensor:
     32-row block ``row//32``, d-block ``d//32``, register group ``(d%32)//8``, wave half
     ``(d%8)//4``, lane column ``row%32``, component ``d%4``."""
     B, H, N, D = Acc_frag.shape
-    v = Acc_frag.view(B, H, N // 32, 4, 4, 2, 32, 4)  # rb, db, rg, half, q, c
+    v = Acc_frag.view(B, H, N // 32, D // 32, 4, 2, 32, 4)  # rb, db, rg, half, q, c
     return v.permute(0, 1, 2, 6, 3, 4, 5, 7).reshape(B, H, N, D)
 
 

@@ -42,8 +42,8 @@ int check_common_dims(const Dims& d, const char* who) {
     set_error("%s: n_kv_heads (%d) must divide n_q_heads (%d)", who, d.n_kv_heads, d.n_q_heads);
     return AA_EBADARG;
   }
-  if (d.head_dim != 128) {
-    set_error("%s: head_dim %d is not supported (only 128)", who, d.head_dim);
+  if (d.head_dim != 128 && d.head_dim != 64) {
+    set_error("%s: head_dim %d is not supported (128 or 64)", who, d.head_dim);
     return AA_EUNSUPPORTED;
   }
   if (d.n_ctx % 128 != 0) {
@@ -79,7 +79,7 @@ int check_dims(const Dims& d, const char* who) {
   return AA_OK;
 }
 
-int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, int n_ctx, const char* who, const char* name) {
+int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, int n_ctx, int head_dim, const char* who, const char* name) {
   if (ptr == nullptr) {
     set_error("%s: %s is NULL", who, name);
     return AA_EBADARG;
@@ -88,7 +88,7 @@ int check_tensor(const void* ptr, int64_t sb, int64_t sh, int64_t sn, int n_ctx,
     set_error("%s: %s must be 16-byte aligned with strides that are multiples of 8 elements (ptr=%p strides=%lld,%lld,%lld)", who, name, ptr, (long long)sb, (long long)sh, (long long)sn);
     return AA_EMISALIGNED;
   }
-  if (sn < 128) {
+  if (sn < head_dim) {
     set_error("%s: %s row stride %lld is smaller than head_dim", who, name, (long long)sn);
     return AA_EBADARG;
   }
@@ -168,14 +168,14 @@ struct Workspace {
   size_t M, L, acc, qbar, abar, mask, coords, counts, total;
 };
 
-Workspace carve(int batch, int hq, int n_ctx, int block_size, int step) {
+Workspace carve(int batch, int hq, int n_ctx, int head_dim, int block_size, int step) {
   Workspace w;
   const size_t bh = (size_t)batch * hq;
   size_t off = 0;
   w.M = off;      off += align256(bh * n_ctx * 4);
   w.L = off;      off += align256(bh * n_ctx * 4);
-  w.acc = off;    off += align256(bh * n_ctx * 128 * 4);
-  w.qbar = off;   off += align256(bh * (n_ctx / block_size) * 128 * 2);
+  w.acc = off;    off += align256(bh * n_ctx * head_dim * 4);
+  w.qbar = off;   off += align256(bh * (n_ctx / block_size) * head_dim * 2);
   w.abar = off;   off += align256(bh * (n_ctx / block_size) * 2);
   w.mask = off;   off += align256((size_t)aa_mask_words(batch, hq, n_ctx, block_size, step) * 4);
   w.coords = off; off += align256(bh * (size_t)aa_coords_entries_per_head(n_ctx, block_size, step) * 4);
@@ -195,7 +195,7 @@ extern "C" {
 #define AA_ABLATE 0
 #endif
 // (1000 + n marks a timing-only build that leaves part of a kernel out, see aa_flash.hip; never a product)
-int aa_version(void) { return AA_ABLATE ? 1000 + AA_ABLATE : 2; }
+int aa_version(void) { return AA_ABLATE ? 1000 + AA_ABLATE : 3; }
 
 const char* aa_last_error(void) { return g_error; }
 
@@ -218,8 +218,8 @@ int64_t aa_mask_words(int batch, int n_q_heads, int n_ctx, int block_size, int s
 }
 
 size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int block_size, int step) {
-  if (batch <= 0 || n_q_heads <= 0 || n_ctx <= 0 || head_dim != 128 || block_size <= 0 || step <= 0) return 0;
-  return carve(batch, n_q_heads, n_ctx, block_size, step).total;
+  if (batch <= 0 || n_q_heads <= 0 || n_ctx <= 0 || (head_dim != 128 && head_dim != 64) || block_size <= 0 || step <= 0) return 0;
+  return carve(batch, n_q_heads, n_ctx, head_dim, block_size, step).total;
 }
 
 // Stage 1; with qbar/abar non-null (block_size <= 128) the kernel also emits the pooled queries and anchors.
@@ -232,9 +232,9 @@ static int stage1_impl(const char* who, const void* q, int64_t q_sb, int64_t q_s
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
   if ((rc = check_dtype(dtype, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, head_dim, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, head_dim, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, head_dim, who, "v"))) return rc;
   if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag"))) return rc;
   if (scale_mode != AA_SCALE_BF16_CHAIN && scale_mode != AA_SCALE_FP32) {
     set_error("%s: unknown scale_mode %d", who, scale_mode);
@@ -246,7 +246,7 @@ static int stage1_impl(const char* who, const void* q, int64_t q_sb, int64_t q_s
   a.v = (const uint16_t*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
   a.M_out = M; a.L_out = L; a.acc_out = acc_frag;
   a.qbar_out = (uint16_t*)qbar; a.abar_out = (uint16_t*)abar;
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx; a.head_dim = head_dim;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = scale_mode; a.dtype = dtype;
   return check_launch(run_flash(a, 0, (hipStream_t)stream), who);
@@ -269,12 +269,12 @@ int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, co
   int rc;
   if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_dims({batch, n_q_heads, n_q_heads, n_ctx, head_dim, block_size, 16}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, head_dim, who, "q"))) return rc;
   if ((rc = check_ptr(M, who, "M")) || (rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar"))) return rc;
   PoolArgs a = {};
   a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
   a.M = M; a.qbar = (uint16_t*)qbar; a.abar = (uint16_t*)abar;
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_ctx = n_ctx; a.block_size = block_size; a.dtype = dtype;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_ctx = n_ctx; a.block_size = block_size; a.head_dim = head_dim; a.dtype = dtype;
   return check_launch(launch_pool(a, (hipStream_t)stream), who);
 }
 
@@ -291,7 +291,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
     return AA_EBADARG;
   }
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, head_dim, who, "k"))) return rc;
   if ((rc = check_ptr(qbar, who, "qbar")) || (rc = check_ptr(abar, who, "abar")) || (rc = check_ptr(mask_ws, who, "mask_ws")) ||
       (rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")))
     return rc;
@@ -301,7 +301,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
   a.mask = mask_ws; a.coords = coords; a.counts = counts;
   a.thr = reinterpret_cast<float*>(mask_ws + mask_bit_words(batch, n_q_heads, n_ctx, block_size, step));
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx; a.head_dim = head_dim;
   a.big_block = block_size * step; a.block_size = block_size;
   a.scale2 = (float)(sm_scale * 1.44269504);  // double product, then float32, as the definition does
   a.theta_log2 = theta_log2;
@@ -311,7 +311,7 @@ int aa_stage2_select(const void* qbar, const void* abar,
   // the score kernel numbers (query head of the KV group, big block) pairs with 16 bits and addresses the pooled
   // queries with 32-bit byte offsets
   if ((int64_t)(n_q_heads / n_kv_heads) * (n_ctx / (block_size * step)) >= 65536 ||
-      (int64_t)batch * n_q_heads * (n_ctx / block_size) * 256 > 0xffffffffLL) {
+      (int64_t)batch * n_q_heads * (n_ctx / block_size) * 2 * head_dim > 0xffffffffLL) {
     set_error("%s: too many (head, big block) pairs or pooled rows for one launch (heads per KV head %d, big blocks %d, pooled rows %lld)",
               who, n_q_heads / n_kv_heads, n_ctx / (block_size * step), (long long)batch * n_q_heads * (n_ctx / block_size));
     return AA_EUNSUPPORTED;
@@ -354,10 +354,10 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   int rc;
   if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
-  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, who, "out"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, head_dim, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, head_dim, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, head_dim, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, head_dim, who, "out"))) return rc;
   if ((rc = check_ptr(coords, who, "coords")) || (rc = check_ptr(counts, who, "counts")) || (rc = check_ptr(M, who, "M")) ||
       (rc = check_ptr(L, who, "L")) || (rc = check_ptr(acc_frag, who, "acc_frag")))
     return rc;
@@ -369,7 +369,7 @@ int aa_stage3_sparse_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
   a.M = M; a.L = L; a.acc_frag = acc_frag;
   a.coords = coords; a.counts = counts;
   a.coords_per_head = aa_coords_entries_per_head(n_ctx, block_size, step);
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx; a.head_dim = head_dim;
   a.big_block = block_size * step; a.block_size = block_size;
   a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32; a.dtype = dtype;
   return check_launch(run_flash(a, 1, (hipStream_t)stream), who);
@@ -387,7 +387,7 @@ int aa_anchor_attn_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   int rc;
   if ((rc = check_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, block_size, step}, who))) return rc;
   if ((rc = check_ptr(workspace, who, "workspace"))) return rc;
-  const Workspace w = carve(batch, n_q_heads, n_ctx, block_size, step);
+  const Workspace w = carve(batch, n_q_heads, n_ctx, head_dim, block_size, step);
   if (workspace_bytes < w.total) {
     set_error("%s: workspace has %zu bytes, %zu needed", who, workspace_bytes, w.total);
     return AA_EBADARG;
@@ -436,16 +436,16 @@ int aa_dense_causal_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
   int rc;
   if ((rc = check_dtype(dtype, who))) return rc;
   if ((rc = check_common_dims({batch, n_q_heads, n_kv_heads, n_ctx, head_dim, 128, 16}, who))) return rc;
-  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, who, "q"))) return rc;
-  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, who, "k"))) return rc;
-  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, who, "v"))) return rc;
-  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, who, "out"))) return rc;
+  if ((rc = check_tensor(q, q_sb, q_sh, q_sn, n_ctx, head_dim, who, "q"))) return rc;
+  if ((rc = check_tensor(k, k_sb, k_sh, k_sn, n_ctx, head_dim, who, "k"))) return rc;
+  if ((rc = check_tensor(v, v_sb, v_sh, v_sn, n_ctx, head_dim, who, "v"))) return rc;
+  if ((rc = check_tensor(out, o_sb, o_sh, o_sn, n_ctx, head_dim, who, "out"))) return rc;
   FlashArgs a = {};
   a.q = (const uint16_t*)q; a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn;
   a.k = (const uint16_t*)k; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.v = (const uint16_t*)v; a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn;
   a.out = (uint16_t*)out; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
-  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx;
+  a.batch = batch; a.n_q_heads = n_q_heads; a.n_kv_heads = n_kv_heads; a.n_ctx = n_ctx; a.head_dim = head_dim;
   a.big_block = n_ctx; a.block_size = 128;  // one "big block": bb is always 0
   a.sm_scale = sm_scale; a.scale_mode = AA_SCALE_FP32; a.dtype = dtype;
   return check_launch(run_flash(a, 2, (hipStream_t)stream), who);

@@ -44,7 +44,6 @@ namespace aa {
 constexpr int kBN = 64;        // keys per LDS tile
 constexpr int kRowBytes = 256;   // one K/V row in LDS (128 bf16, unpadded, chunks swizzled)
 constexpr int kTileBytes = kBN * kRowBytes;
-constexpr int kOsStride = 136;   // bf16 per output-staging row in LDS
 constexpr int kDist = 4;         // MFMA operands are fetched from LDS this many MFMAs ahead of their use
 constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
 
@@ -76,7 +75,7 @@ struct FlashSmem {
       char k[2][kTileBytes];
       char v[2][kTileBytes];
     } t;
-    uint16_t os[4][32 * kOsStride];  // epilogue staging, reuses the tile space
+    uint16_t os[4][32 * 136];  // epilogue staging (row stride D + 8 elements), reuses the tile space
   };
   int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
 };
@@ -139,12 +138,22 @@ __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, cons
   }
 }
 
-template <int MODE, typename T>
+// D is the head dimension, 128 or 64.  With 64 the LDS tiles keep their 256-byte row pitch and their swizzles - a row
+// then fills eight of its sixteen 16-byte slots, the lanes of a tile load that would bring the other eight fetch a
+// duplicate that is never read - so every LDS address below is the same for both sizes, and only the number of MFMA steps
+// over the head dimension (kKS per 32 keys of Q.K^T) and of 32-column output blocks (kDB) changes.
+template <int MODE, typename T, int D>
 __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   typedef typename T::vec8 vec8;
   typedef __attribute__((address_space(3))) vec8 lds_vec8;
   __shared__ __attribute__((aligned(16))) FlashSmem<MODE == kSparse> sm;
   constexpr int BM = 128;
+  static_assert(D == 128 || D == 64, "head dimension");
+  constexpr int kKS = D / 16;       // MFMAs per 32-key block of S^T = K Q^T
+  constexpr int kDB = D / 32;       // 32-column blocks of the head dimension: accumulators of O^T
+  constexpr int kNS = 2 * kKS;      // S^T slots of a 64-key tile
+  constexpr int kNV = 4 * kDB;      // O^T slots of a 64-key tile (two 16-key steps per 32-key block)
+  constexpr int kOsStride = D + 8;  // 16-bit elements per output-staging row in LDS
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -206,13 +215,13 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   // They depend on nothing, whereas the first K/V tile needs the index list, which needs its own round trip to
   // memory.  The 64 KB of accumulator state follow the first tile's loads (further down) and are not waited for
   // before the first scores are computed.
-  u32x4 qraw[8];
+  u32x4 qraw[kKS];
   float m_run, l_run;
-  floatx16 acc[4];
+  floatx16 acc[kDB];
   const uint16_t* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
   if (MODE == kSparse) {
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
+    for (int ks = 0; ks < kKS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
     m_run = p.M[bh * p.n_ctx + my_row];
     l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
   }
@@ -265,15 +274,16 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   }
 
   // this thread's chunk of a row (swizzled: see the top of the file) and the wave's slice of the LDS tiles
-  const uint32_t k_col = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15)) * 16u;
-  const uint32_t v_col = (uint32_t)((tid & 15) ^ (((tid >> 4) & 7) << 1)) * 16u;
+  // (head dimension 64: a row has eight chunks; the lanes whose slot belongs to none of them fetch a duplicate)
+  const uint32_t k_col = (uint32_t)(((tid & 15) ^ ((tid >> 4) & 15)) & (D / 8 - 1)) * 16u;
+  const uint32_t v_col = (uint32_t)(((tid & 15) ^ (((tid >> 4) & 7) << 1)) & (D / 8 - 1)) * 16u;
   const uint32_t lds_k0 = lds_addr(sm.t.k[0]) + wave * 4 * kRowBytes, lds_v0 = lds_addr(sm.t.v[0]) + wave * 4 * kRowBytes;
   // byte offset of this thread's chunk of row (tid >> 4) of a block of 16 tile rows from the block's first row
   const uint32_t k_voff = (tid >> 4) * k_row_bytes + k_col, v_voff = (tid >> 4) * v_row_bytes + v_col;
   // (anchor mode with pooling) the work-group's raw query rows, fetched like a tile by the last tile's load slots
   const char* qblock = reinterpret_cast<const char*>(qp + (int64_t)R0 * p.q_sn);
   const uint32_t q_row_bytes = (uint32_t)p.q_sn * 2u;
-  const uint32_t q_voff = (uint32_t)(tid >> 4) * q_row_bytes + (uint32_t)(tid & 15) * 16u;
+  const uint32_t q_voff = (uint32_t)(tid >> 4) * q_row_bytes + (uint32_t)((tid & 15) & (D / 8 - 1)) * 16u;
   if (n_tiles > 0) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
@@ -284,9 +294,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // the accumulator state: the youngest loads in flight, first needed by the first P.V product.  (The accumulator
     // state and the output are touched once each: they are written and read with the non-temporal hint, so that they
     // do not push K/V rows, which many work-groups share, out of the L2.)
-    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
+    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * (4 * kDB)) * 256 + lane * 4;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < kDB; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         floatx4 t = {0.f, 0.f, 0.f, 0.f};
@@ -297,15 +307,15 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   }
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
-  vec8 qreg[8];
+  vec8 qreg[kKS];
   {
     const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
     if (MODE != kSparse) {
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
+      for (int ks = 0; ks < kKS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qreg[ks] = scale_q8<T>(qraw[ks], p.sm_scale, chain);
+    for (int ks = 0; ks < kKS; ++ks) qreg[ks] = scale_q8<T>(qraw[ks], p.sm_scale, chain);
   }
 
   // ---- running state (sparse mode loaded it at the top) -----------------------------------------
@@ -313,7 +323,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     m_run = -INFINITY;
     l_run = 0.f;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < kDB; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
   }
@@ -326,10 +336,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   for (int r = 0; r < 16; ++r) negm[r] = -m_ref;
 
   if (MODE == kSparse) {
-    // Loads complete in order and 64 registers take at least 16 load instructions, so "at most 16 outstanding" means:
-    // everything requested before the accumulator state - queries, statistics, tile 0 - has arrived.  The state
-    // itself may still be on its way while the first scores are computed (the compiler waits where it is first used).
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    // Loads complete in order and the accumulator state was requested last, with 4 * kDB load instructions, so "at most
+    // that many outstanding" means: everything requested before it - queries, statistics, tile 0 - has arrived.  The
+    // state itself may still be on its way while the first scores are computed (the compiler waits where it is first used).
+    if (kDB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     lds_barrier();  // a barrier that does not wait for the loads still in flight
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
@@ -338,18 +349,18 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 
   // per-lane LDS byte offsets.  K: row c32 (+32*kb), chunk 2*ks + half, swizzled with the row's low four bits.
   // (absolute LDS addresses into the current buffer; the 32-key half and the row steps are immediate offsets)
-  uint32_t k_rd[8];
+  uint32_t k_rd[kKS];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  for (int ks = 0; ks < kKS; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
   // transposing V read i: a group of 16 lanes covers 16 head-dim columns; lane points at row r0 = 4*half + (lane%16)/4
   // (+ multiples of 8, which leave r0 = row & 7 alone), bf16 columns 32*(i&3) + 16*((lane>>4)&1) + 4*(lane&3): chunk
   // 4*(i&3) + y0 with y0 < 4, swizzled with r0 << 1 -> one offset per value of i & 3
-  uint32_t v_rd[4];
+  uint32_t v_rd[kDB];
   {
     const int r0 = 4 * half + ((lane & 15) >> 2);
     const int y0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
+    for (int m = 0; m < kDB; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
   }
 
 
@@ -387,8 +398,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     pw[(c) >> 1][2 * ((c) & 1) + 0] = T::pack(e0, e1);                                 \
     pw[(c) >> 1][2 * ((c) & 1) + 1] = T::pack(e2, e3);                                 \
   }
-  // V operand fetch i (two transposing reads): i = (kb*2 + st)*4 + db
-#define AA_V_SRC(i) (v_rd[(i) & 3] + (uint32_t)(rd_off + (32 * ((i) >> 3) + 16 * (((i) >> 2) & 1)) * kRowBytes))
+  // V operand fetch i (two transposing reads): i = (kb*2 + st)*kDB + db
+#define AA_V_SRC(i) (v_rd[(i) % kDB] + (uint32_t)(rd_off + (32 * ((i) / (2 * kDB)) + 16 * (((i) / kDB) & 1)) * kRowBytes))
 #define AA_V_FETCH(i)                                                                                  \
   {                                                                                                    \
     vlo[i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(AA_V_SRC(i)));                     \
@@ -398,8 +409,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   {                                                                                                    \
     typedef short shortx8 __attribute__((ext_vector_type(8)));                                         \
     const shortx8 av = __builtin_shufflevector(vlo[i], vhi[i], 0, 1, 2, 3, 4, 5, 6, 7);                \
-    acc[(i) & 3] = T::mfma(*reinterpret_cast<const vec8*>(&av),                                        \
-                           AA_ABLATE == 10 ? qreg[(i) & 7] : *reinterpret_cast<const vec8*>(&pw[((i) >> 2) & 1]), acc[(i) & 3]); \
+    acc[(i) % kDB] = T::mfma(*reinterpret_cast<const vec8*>(&av),                                      \
+                             AA_ABLATE == 10 ? qreg[(i) % kKS] : *reinterpret_cast<const vec8*>(&pw[((i) / kDB) & 1]), acc[(i) % kDB]); \
   }
 #define AA_FENCE __builtin_amdgcn_sched_barrier(0)
 
@@ -447,40 +458,46 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // runs it fully masked: it would only wait at the barrier for the others anyway)
     {
       floatx16 s0, s1;
-      vec8 ka[16];              // K operand of slot n = kb*8 + ks
-      shortx4 vlo[16], vhi[16];  // V operand of slot 16 + i, i = (kb*2 + st)*4 + db
-      u32x4 pw0[2], pw1[2];      // P^T fragments (bf16 pairs) of the two halves
+      vec8 ka[kNS];                // K operand of slot n = kb*kKS + ks
+      shortx4 vlo[kNV], vhi[kNV];  // V operand of slot kNS + i, i = (kb*2 + st)*kDB + db
+      u32x4 pw0[2], pw1[2];        // P^T fragments (bf16 pairs) of the two halves
       float mx0, mx1, sum0 = 0.f, sum1 = 0.f, shift0 = 0.f, alpha1 = 1.f;
-#define AA_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) & 7] + (uint32_t)(rd_off + 32 * ((t) >> 3) * kRowBytes))
+#define AA_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) % kKS] + (uint32_t)(rd_off + 32 * ((t) / kKS) * kRowBytes))
 
-      // The 32 MFMAs of a tile are slots 0..31 (16 for S^T, 16 for O^T); the operand of slot n is fetched from
-      // LDS while slot n - kDist is issued.  The scheduling fences keep that distance: left alone, the reads sink
-      // next to their use and every MFMA then waits out a full LDS latency.
+      // The MFMAs of a tile are slots 0 .. kNS + kNV - 1 (head dimension 128: 16 for S^T, then 16 for O^T); the operand of
+      // slot n is fetched from LDS while slot n - kDist is issued.  The scheduling fences keep that distance: left
+      // alone, the reads sink next to their use and every MFMA then waits out a full LDS latency.
 #define AA_OPERAND_FETCH(n)                          \
   {                                                  \
-    if ((n) < 16) {                                  \
-      AA_K_FETCH((n) & 15);                          \
-    } else if ((n) < 32) {                           \
-      AA_V_FETCH(((n) - 16) & 15)                    \
+    if ((n) < kNS) {                                 \
+      AA_K_FETCH((n) % kNS);                         \
+    } else if ((n) < kNS + kNV) {                    \
+      AA_V_FETCH(((n) - kNS) % kNV)                  \
     }                                                \
   }
-#define AA_S_MFMA(sx, n) sx = T::mfma(ka[n], qreg[(n) & 7], ((n) & 7) == 0 ? negm : sx)
+#define AA_S_MFMA(sx, n) sx = T::mfma(ka[n], qreg[(n) % kKS], ((n) % kKS) == 0 ? negm : sx)
+      // Each half-tile product is kKS (S^T) or 2*kDB (O^T) MFMAs long; the soft-max of the other half sits between them:
+      // a quarter of the MFMAs, the row max, half of the MFMAs with the four exp chunks spread over them, the last quarter.
+      constexpr int kSPre = kKS / 4, kSMid = kKS / 2, kVPre = kDB / 2, kVMid = kDB;
 #pragma unroll
       for (int n = 0; n < kDist; ++n) AA_OPERAND_FETCH(n)
       AA_FENCE;
 
       // ---- phase A: S0^T = K0 Q^T (and the next tile's eight loads) -------------------------------
 #pragma unroll
-      for (int n = 0; n < 8; ++n) {
+      for (int n = 0; n < kKS; ++n) {
         AA_OPERAND_FETCH(n + kDist)
         AA_S_MFMA(s0, n);
-        if (AA_ABLATE != 3) { AA_FETCH_ONE(n) }
+        if (AA_ABLATE != 3) {
+#pragma unroll
+          for (int u = 0; u < 8 / kKS; ++u) { AA_FETCH_ONE(n * (8 / kKS) + u) }
+        }
         AA_FENCE;
       }
 
       // ---- phase B: S1^T = K1 Q^T, with the soft-max of S0 between the MFMAs ---------------------
 #pragma unroll
-      for (int n = 8; n < 10; ++n) {
+      for (int n = kKS; n < kKS + kSPre; ++n) {
         AA_OPERAND_FETCH(n + kDist)
         AA_S_MFMA(s1, n);
         AA_FENCE;
@@ -506,21 +523,22 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) negm[r] = -m_new;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDB; ++db)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
       }
       AA_FENCE;
 #pragma unroll
-      for (int n = 10; n < 14; ++n) {
+      for (int n = kKS + kSPre; n < kKS + kSPre + kSMid; ++n) {
         AA_OPERAND_FETCH(n + kDist)
         AA_S_MFMA(s1, n);
-        AA_EXP_CHUNK(s0, pw0, sum0, n - 10)
+#pragma unroll
+        for (int u = 0; u < 4 / kSMid; ++u) { AA_EXP_CHUNK(s0, pw0, sum0, (n - kKS - kSPre) * (4 / kSMid) + u) }
         AA_FENCE;
       }
       l_run += sum0;
 #pragma unroll
-      for (int n = 14; n < 16; ++n) {
+      for (int n = kKS + kSPre + kSMid; n < kNS; ++n) {
         AA_OPERAND_FETCH(n + kDist)
         AA_S_MFMA(s1, n);
         AA_FENCE;
@@ -528,9 +546,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 
       // ---- phase C: O^T += V0^T P0^T, with the soft-max of S1 between the MFMAs --------------------
 #pragma unroll
-      for (int n = 16; n < 18; ++n) {
+      for (int n = kNS; n < kNS + kVPre; ++n) {
         AA_OPERAND_FETCH(n + kDist)
-        AA_PV_MFMA(n - 16, pw0)
+        AA_PV_MFMA(n - kNS, pw0)
         AA_FENCE;
       }
       if (moved0) {
@@ -559,31 +577,32 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
       AA_FENCE;
 #pragma unroll
-      for (int n = 18; n < 22; ++n) {
+      for (int n = kNS + kVPre; n < kNS + kVPre + kVMid; ++n) {
         AA_OPERAND_FETCH(n + kDist)
-        AA_PV_MFMA(n - 16, pw0)
-        AA_EXP_CHUNK(s1, pw1, sum1, n - 18)
+        AA_PV_MFMA(n - kNS, pw0)
+#pragma unroll
+        for (int u = 0; u < 4 / kVMid; ++u) { AA_EXP_CHUNK(s1, pw1, sum1, (n - kNS - kVPre) * (4 / kVMid) + u) }
         AA_FENCE;
       }
       l_run += sum1;
 #pragma unroll
-      for (int n = 22; n < 24; ++n) {
+      for (int n = kNS + kVPre + kVMid; n < kNS + 2 * kDB; ++n) {
         AA_OPERAND_FETCH(n + kDist)
-        AA_PV_MFMA(n - 16, pw0)
+        AA_PV_MFMA(n - kNS, pw0)
         AA_FENCE;
       }
       if (moved1) {
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDB; ++db)
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[db][r] *= alpha1;
       }
 
       // ---- phase D: O^T += V1^T P1^T ---------------------------------------------------------------
 #pragma unroll
-      for (int n = 24; n < 32; ++n) {
+      for (int n = kNS + 2 * kDB; n < kNS + kNV; ++n) {
         AA_OPERAND_FETCH(n + kDist)
-        AA_PV_MFMA(n - 16, pw1)
+        AA_PV_MFMA(n - kNS, pw1)
         AA_FENCE;
       }
       if (AA_ABLATE == 10) {  // P is still formed: it only has to exist by the end of the tile
@@ -597,9 +616,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 
     if (kBuf < 0) {  // the read addresses follow the tiles into the other buffer
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) k_rd[ks] += buf_step;
+      for (int ks = 0; ks < kKS; ++ks) k_rd[ks] += buf_step;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) v_rd[m] += buf_step;
+      for (int m = 0; m < kDB; ++m) v_rd[m] += buf_step;
       buf_step = -buf_step;
     }
     if (AA_ABLATE != 9) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
@@ -631,9 +650,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       p.M_out[bh * p.n_ctx + my_row] = m_run;
       p.L_out[bh * p.n_ctx + my_row] = l_tot;
     }
-    float* af = p.acc_out + ((bh * (p.n_ctx / 32) + my_row / 32) * 16) * 256 + lane * 4;
+    float* af = p.acc_out + ((bh * (p.n_ctx / 32) + my_row / 32) * (4 * kDB)) * 256 + lane * 4;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < kDB; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         floatx4 t;
@@ -652,7 +671,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       const int bs = p.block_size, n_pooled = BM / bs;  // pooled rows of this work-group (1 for block_size 128)
       const int n_pr = p.n_ctx / bs;
       const float d = (float)bs;
-      if (tid < 128) {
+      if (tid < D) {
         // waves 0 and 1: one head-dim column per thread (the ordered sum is a serial chain per column, so the shorter
         // the chain per thread the sooner the work-group retires)
         for (int pp = 0; pp < n_pooled; ++pp) {
@@ -665,9 +684,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
             for (int t = 0; t < 16; ++t) a0 += T::from16(w[t]);
           }
-          reinterpret_cast<uint16_t*>(p.qbar_out)[((bh * n_pr) + R0 / bs + pp) * 128 + tid] = (uint16_t)(T::pack(a0 / d, 0.f) & 0xffffu);
+          reinterpret_cast<uint16_t*>(p.qbar_out)[((bh * n_pr) + R0 / bs + pp) * D + tid] = (uint16_t)(T::pack(a0 / d, 0.f) & 0xffffu);
         }
-      } else if (tid - 128 < n_pooled) {
+      } else if (tid >= 128 && tid - 128 < n_pooled) {
         // meanwhile, in wave 2: one thread per pooled anchor
         const int pp = tid - 128;
         float am = 0.f;
@@ -682,11 +701,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
     }
   } else {
-    // out = bf16(acc / l): stage the wave's [32][128] tile in LDS, then write whole rows
+    // out = bf16(acc / l): stage the wave's [32][D] tile in LDS, then write whole rows
     uint16_t* os = sm.os[wave];
     const float inv = 1.0f / l_tot;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < kDB; ++db)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         u32x2 w;
@@ -696,9 +715,10 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
     __syncthreads();
     uint16_t* op = p.out + b * p.o_sb + hq * p.o_sh;
+    constexpr int kLanesPerRow = D / 8, kRowsPerStore = 64 / kLanesPerRow;  // a row is D/8 pieces of 16 bytes
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int r = it * 4 + (lane >> 4), c = lane & 15;
+    for (int it = 0; it < 32 / kRowsPerStore; ++it) {
+      const int r = it * kRowsPerStore + lane / kLanesPerRow, c = lane % kLanesPerRow;
       const u32x4 w = *reinterpret_cast<const u32x4*>(&os[r * kOsStride + 8 * c]);
       __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c));
     }
@@ -720,9 +740,14 @@ static hipError_t launch(const FlashArgs& args, hipStream_t stream) {
     const int per_big_block = a.big_block / 128;  // even for every supported geometry
     a.q_blocks_per_wg = per_big_block % AA_SPARSE_QBLOCKS == 0 ? AA_SPARSE_QBLOCKS : (per_big_block % 2 == 0 ? 2 : 1);
   }
-  const uint32_t grid = (uint32_t)a.batch * a.n_q_heads * (a.n_ctx / (128 * a.q_blocks_per_wg));
-  if (a.dtype == 0) hipLaunchKernelGGL((flash_kernel<MODE, Bf16>), dim3(grid), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((flash_kernel<MODE, F16>), dim3(grid), dim3(256), 0, stream, a);
+  const dim3 grid((uint32_t)a.batch * a.n_q_heads * (a.n_ctx / (128 * a.q_blocks_per_wg))), block(256);
+  if (a.head_dim == 128) {
+    if (a.dtype == 0) hipLaunchKernelGGL((flash_kernel<MODE, Bf16, 128>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((flash_kernel<MODE, F16, 128>), grid, block, 0, stream, a);
+  } else {  // 64: the C-ABI layer admits nothing else
+    if (a.dtype == 0) hipLaunchKernelGGL((flash_kernel<MODE, Bf16, 64>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((flash_kernel<MODE, F16, 64>), grid, block, 0, stream, a);
+  }
   return hipGetLastError();
 }
 

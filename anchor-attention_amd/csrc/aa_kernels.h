@@ -11,11 +11,12 @@ struct FlashArgs {
   uint16_t* out;     int64_t o_sb, o_sh, o_sn;   // sparse / dense modes
   float* M_out; float* L_out; float* acc_out;  // anchor mode
   // anchor mode, optional (both or neither; block_size <= 128): the work-group also mean-pools its 128 raw query rows
-  // and anchors into qbar [B,Hq,N/block_size,128] and abar [B,Hq,N/block_size], bit for bit what pool_kernel computes
+  // and anchors into qbar [B,Hq,N/block_size,head_dim] and abar [B,Hq,N/block_size], bit for bit what pool_kernel computes
   uint16_t* qbar_out; uint16_t* abar_out;
   const float* M; const float* L; const float* acc_frag;  // sparse mode (resume state)
   const int32_t* coords; const int32_t* counts; int64_t coords_per_head;  // sparse mode
   int batch, n_q_heads, n_kv_heads, n_ctx;
+  int head_dim;  // 128 or 64
   int big_block, block_size;
   float sm_scale; int scale_mode;
   int q_blocks_per_wg;  // set by the launcher
@@ -30,6 +31,7 @@ struct PoolArgs {
   const float* M;
   uint16_t* qbar; uint16_t* abar;
   int batch, n_q_heads, n_ctx, block_size;
+  int head_dim;  // 128 or 64
   int dtype;
 };
 hipError_t launch_pool(const PoolArgs& a, hipStream_t stream);
@@ -44,6 +46,7 @@ struct SelectArgs {
   float scale2, theta_log2;
   // candidate keys of big block bb: key_lo <= j < bb*S - key_slack (as run: block_size and block_size; intended: S and 0)
   int key_lo, key_slack;
+  int head_dim;  // 128 or 64
   int dtype;
 };
 hipError_t launch_select_thresholds(const SelectArgs& a, hipStream_t stream);

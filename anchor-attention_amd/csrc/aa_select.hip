@@ -23,12 +23,14 @@
 namespace aa {
 
 // ------------------------------------------------------------------------------------------------
-template <typename T>
+// D = head dimension (128 or 64): D/8 lanes of 16 bytes cover a query row, a wave pools 64 / (D/8) blocks.
+template <typename T, int D>
 __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
+  constexpr int kLanesPerRow = D / 8, kBlocksPerWave = 64 / kLanesPerRow;
   const int lane = threadIdx.x;
-  const int c = lane & 15;
+  const int c = lane % kLanesPerRow;
   const int n_pr = p.n_ctx / p.block_size;
-  const int pr = 4 * blockIdx.x + (lane >> 4);
+  const int pr = kBlocksPerWave * blockIdx.x + lane / kLanesPerRow;
   const int h = blockIdx.y, b = blockIdx.z;
   if (pr >= n_pr) return;
   const int bs = p.block_size;
@@ -52,7 +54,7 @@ __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
   o.y = T::pack(acc[2] / d, acc[3] / d);
   o.z = T::pack(acc[4] / d, acc[5] / d);
   o.w = T::pack(acc[6] / d, acc[7] / d);
-  *reinterpret_cast<uint4*>(p.qbar + (bh * n_pr + pr) * 128 + 8 * c) = o;
+  *reinterpret_cast<uint4*>(p.qbar + (bh * n_pr + pr) * D + 8 * c) = o;
   if (c == 0) {
     const uint32_t w = T::pack(am / d, 0.f);
     reinterpret_cast<uint16_t*>(p.abar)[bh * n_pr + pr] = (uint16_t)(w & 0xffffu);
@@ -61,8 +63,15 @@ __global__ void __launch_bounds__(64) pool_kernel(const PoolArgs p) {
 
 hipError_t launch_pool(const PoolArgs& a, hipStream_t stream) {
   const int n_pr = a.n_ctx / a.block_size;
-  if (a.dtype == 0) hipLaunchKernelGGL(pool_kernel<Bf16>, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
-  else hipLaunchKernelGGL(pool_kernel<F16>, dim3((n_pr + 3) / 4, a.n_q_heads, a.batch), dim3(64), 0, stream, a);
+  const int per_wave = a.head_dim == 128 ? 4 : 8;
+  const dim3 grid((n_pr + per_wave - 1) / per_wave, a.n_q_heads, a.batch);
+  if (a.head_dim == 128) {
+    if (a.dtype == 0) hipLaunchKernelGGL((pool_kernel<Bf16, 128>), grid, dim3(64), 0, stream, a);
+    else hipLaunchKernelGGL((pool_kernel<F16, 128>), grid, dim3(64), 0, stream, a);
+  } else {
+    if (a.dtype == 0) hipLaunchKernelGGL((pool_kernel<Bf16, 64>), grid, dim3(64), 0, stream, a);
+    else hipLaunchKernelGGL((pool_kernel<F16, 64>), grid, dim3(64), 0, stream, a);
+  }
   return hipGetLastError();
 }
 
@@ -144,8 +153,12 @@ __device__ __forceinline__ void sel_load4_to_lds(const char* base, const uint32_
   asm volatile("s_nop 0\n\tglobal_load_lds_dword %1, %2" : : "{m0}"(lds_dst), "v"(byte_off), "s"(base) : "memory");
 }
 
-template <int STEP, int WAVES, int ROWS, typename T>
+// D = head dimension (128 or 64).  With 64 the pooled rows keep their 256-byte pitch in LDS: a row fills eight of its
+// sixteen 16-byte slots (the staging lanes whose slot belongs to no chunk fetch a duplicate that is never read), so
+// the LDS addressing is that of 128 and only the number of MFMA steps over the head dimension changes.
+template <int STEP, int WAVES, int ROWS, typename T, int D>
 __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(const SelectArgs p) {
+  constexpr int kKS = D / 16;                    // MFMA steps over the head dimension
   constexpr int kItems = 32 / STEP;              // items per 32-row MFMA group
   constexpr int kGroups = ROWS / 32;             // MFMA groups per block
   constexpr int kBlockItems = ROWS / STEP;       // items per block
@@ -198,12 +211,12 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
 
   typedef typename T::vec8 vec8;
   const uint16_t* kp = p.k + b * p.k_sb + kvh * p.k_sh;
-  vec8 kreg[kKB][8];
+  vec8 kreg[kKB][kKS];
 #pragma unroll
   for (int kb = 0; kb < kKB; ++kb) {
     const uint16_t* row = kp + (int64_t)(tw * 128 + 32 * (kb0 + kb) + c32) * p.k_sn + 8 * half;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) kreg[kb][ks] = *reinterpret_cast<const vec8*>(row + 16 * ks);
+    for (int ks = 0; ks < kKS; ++ks) kreg[kb][ks] = *reinterpret_cast<const vec8*>(row + 16 * ks);
   }
 
   // ---- staging -------------------------------------------------------------------------------
@@ -227,8 +240,8 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
     for (int j = 0; j < kRowsPerWave / 4; ++j) {
       const int r = 4 * j + (lane >> 4);  // row inside the wave's share
       const uint32_t prow = item_row0[r / STEP] + (uint32_t)(r % STEP);
-      const uint32_t chunk = (uint32_t)((lane & 15) ^ (r & 15));
-      sel_load16_to_lds(qbar_base, prow * (uint32_t)kSelRowBytes + chunk * 16u, a_lds0 + buf * (ROWS * kSelRowBytes) + 4 * j * kSelRowBytes);
+      const uint32_t chunk = (uint32_t)(((lane & 15) ^ (r & 15)) & (D / 8 - 1));
+      sel_load16_to_lds(qbar_base, prow * (uint32_t)(2 * D) + chunk * 16u, a_lds0 + buf * (ROWS * kSelRowBytes) + 4 * j * kSelRowBytes);
     }
     if (wave < ROWS / 64) {  // thresholds of block rows 64*wave + lane
       const int r = 64 * wave + lane;
@@ -240,9 +253,9 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   stage_block(0, 0);
 
   // A operand of MFMA step ks: row c32 of the group, chunk 2*ks + half, swizzled with the row's low four bits
-  uint32_t a_rd[8];
+  uint32_t a_rd[kKS];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) a_rd[ks] = sel_lds_addr(a_lds[0]) + c32 * kSelRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  for (int ks = 0; ks < kKS; ++ks) a_rd[ks] = sel_lds_addr(a_lds[0]) + c32 * kSelRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
   typedef __attribute__((address_space(3))) vec8 lds_vec8_t;
   typedef __attribute__((address_space(3))) floatx4 lds_floatx4_t;
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -260,9 +273,9 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
     uint32_t w_lo = 0u, w_hi = 0u;
 #pragma unroll
     for (int gi = 0; gi < kGroups; ++gi) {
-      vec8 a[8];
+      vec8 a[kKS];
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) a[ks] = *(const lds_vec8_t*)(uintptr_t)(a_rd[ks] + a_off + gi * 32 * kSelRowBytes);
+      for (int ks = 0; ks < kKS; ++ks) a[ks] = *(const lds_vec8_t*)(uintptr_t)(a_rd[ks] + a_off + gi * 32 * kSelRowBytes);
       // raw-score thresholds of the accumulator rows this lane holds: row i = 8*(r/4) + 4*half + r%4
       float thr[16];
 #pragma unroll
@@ -276,7 +289,7 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb) c[kb] = T::mfma(a[0], kreg[kb][0], zero);
 #pragma unroll
-      for (int ks = 1; ks < 8; ++ks)
+      for (int ks = 1; ks < kKS; ++ks)
 #pragma unroll
         for (int kb = 0; kb < kKB; ++kb) c[kb] = T::mfma(a[ks], kreg[kb][ks], c[kb]);
 #pragma unroll
@@ -309,16 +322,22 @@ __global__ void __launch_bounds__(64 * WAVES, AA_SEL_WGS) select_scores_kernel(c
   }
 }
 
-hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
+template <typename T, int D>
+static void launch_select_scores_for(const SelectArgs& a, hipStream_t stream) {
   constexpr int kWaves = AA_SEL_WAVES, kRows = AA_SEL_ROWS;
   const int step = a.big_block / a.block_size;
   const dim3 grid((uint32_t)(a.n_ctx / (64 * kWaves)) * a.n_kv_heads * a.batch);
-  if (a.dtype == 0) {
-    if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows, Bf16>), grid, dim3(64 * kWaves), 0, stream, a);
-    else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows, Bf16>), grid, dim3(64 * kWaves), 0, stream, a);
+  if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows, T, D>), grid, dim3(64 * kWaves), 0, stream, a);
+  else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows, T, D>), grid, dim3(64 * kWaves), 0, stream, a);
+}
+
+hipError_t launch_select_scores(const SelectArgs& a, hipStream_t stream) {
+  if (a.head_dim == 128) {
+    if (a.dtype == 0) launch_select_scores_for<Bf16, 128>(a, stream);
+    else launch_select_scores_for<F16, 128>(a, stream);
   } else {
-    if (step == 16) hipLaunchKernelGGL((select_scores_kernel<16, kWaves, kRows, F16>), grid, dim3(64 * kWaves), 0, stream, a);
-    else hipLaunchKernelGGL((select_scores_kernel<32, kWaves, kRows, F16>), grid, dim3(64 * kWaves), 0, stream, a);
+    if (a.dtype == 0) launch_select_scores_for<Bf16, 64>(a, stream);
+    else launch_select_scores_for<F16, 64>(a, stream);
   }
   return hipGetLastError();
 }

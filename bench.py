@@ -32,12 +32,19 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 WORKLOADS = {
-    # name: (n_ctx, hq, hkv, rope_base, n_stripes, stripe_dist)
+    # name: (n_ctx, hq, hkv, rope_base, n_stripes, stripe_dist[, head_dim = 128])
     "config0_llama8b_4k": (4096, 32, 8, 5e5, 64, "uniform"),
     "config1_llama8b_32k": (32768, 32, 8, 5e5, 512, "uniform"),
     "config2_llama8b_128k": (131072, 32, 8, 5e5, 655, "powerlaw"),
     "config3_qwen7b_64k": (65536, 28, 4, 1e6, 328, "uniform"),
+    # not a BASELINE configuration: the Llama-3.2-1B layer shape, for the kernels' head-dimension-64 instantiation
+    "llama1b_128k_headdim64": (131072, 32, 8, 5e5, 655, "powerlaw", 64),
 }
+
+
+def workload_head_dim(name):
+    w = WORKLOADS[name]
+    return w[6] if len(w) > 6 else 128
 
 
 def flops(hq, n_ctx, sum_counts, D=128, S=2048):
@@ -54,8 +61,8 @@ def make_inputs(name, seed, qbar_mode, device):
     is 0.5 G random numbers per tensor); stripe positions still come from the CPU generator."""
     import torch
     from anchor_attn.synthetic import stripe_positions
-    n_ctx, hq, hkv, base, n_stripes, dist = WORKLOADS[name]
-    D = 128
+    n_ctx, hq, hkv, base, n_stripes, dist = WORKLOADS[name][:6]
+    D = workload_head_dim(name)
     g = torch.Generator(device=device).manual_seed(seed)
     cg = torch.Generator(device="cpu").manual_seed(seed)
     inv = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float64, device=device) / D))
@@ -238,8 +245,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    n_ctx, hq, hkv, _, _, _ = WORKLOADS[args.workload]
-    D, BS, STEP, S = 128, 128, 16, 2048
+    n_ctx, hq, hkv = WORKLOADS[args.workload][:3]
+    D, BS, STEP, S = workload_head_dim(args.workload), 128, 16, 2048
     q, k, v = make_inputs(args.workload, args.seed, args.qbar_mode, dev)
     if args.dtype == "fp16":
         q, k, v = q.to(torch.float16), k.to(torch.float16), v.to(torch.float16)
@@ -264,7 +271,7 @@ def main():
 
     # ---- same kernels, staged, with events between them on the launch stream -------------------
     st_ms, sum_counts = staged_pass(q, k, v, args.theta, args.steps, out)
-    f1, f2, f3 = flops(hq, n_ctx, sum_counts)
+    f1, f2, f3 = flops(hq, n_ctx, sum_counts, D=D)
     ratio = sum_counts / ((1 * hq * n_ctx * n_ctx / (BS * STEP)) // 2)
     dense_flops = 4 * D * hq * n_ctx * (n_ctx + 1) / 2
 

@@ -12,7 +12,7 @@
  * h / (n_q_heads / n_kv_heads), the order repeat_kv produces; pass n_kv_heads == n_q_heads for
  * pre-repeated K/V as the reference's caller does).  Element type is bf16 or fp16 (the `dtype`
  * argument, AA_DTYPE_*, the same for every tensor of a call), head_dim must be
- * 128 with stride 1, every row must start on a 16-byte boundary; the other three dimensions
+ * 128 or 64 with stride 1, every row must start on a 16-byte boundary; the other three dimensions
  * are addressed through the element strides (sb, sh, sn), so [B,N,H,D] storage works unchanged.
  * "S" below is the big block, block_size * step keys/queries.
  *
@@ -30,7 +30,7 @@ extern "C" {
 
 #define AA_OK 0
 #define AA_EBADARG 1      /* null pointer, non-positive size, head counts that do not divide, unknown dtype/mode */
-#define AA_EUNSUPPORTED 2 /* head_dim != 128, block_size not in 16..256, step not 16/32, n_ctx % S != 0, n_ctx > 2^20 */
+#define AA_EUNSUPPORTED 2 /* head_dim not 128 or 64, block_size not in 16..256, step not 16/32, n_ctx % S != 0, n_ctx > 2^20 */
 #define AA_EMISALIGNED 3  /* pointer or stride not a multiple of 16 bytes */
 #define AA_ELAUNCH 4      /* HIP runtime error at launch */
 
@@ -84,8 +84,8 @@ size_t aa_workspace_bytes(int batch, int n_q_heads, int n_ctx, int head_dim, int
  * (anchor_step_1_2_v2.py:8-196; call site anchor_attn_v4.py:237-241): flash attention of each
  * query row r over keys [0,S) U [bb*S, r] (bb = r / S), exp2 domain.
  * Outputs: M [B,Hq,N] float32 running max (the anchors), L [B,Hq,N] float32 row sums,
- * acc_frag float32 with B*Hq*N*128 elements: the unnormalised PV accumulator in MFMA fragment
- * order - element (b,h,row,d) lives at ((((b*Hq+h)*(N/32) + row/32)*4 + d/32)*4 + (d%32)/8)*256
+ * acc_frag float32 with B*Hq*N*head_dim elements: the unnormalised PV accumulator in MFMA fragment
+ * order - element (b,h,row,d) lives at ((((b*Hq+h)*(N/32) + row/32)*(head_dim/32) + d/32)*4 + (d%32)/8)*256
  * + (((d%8)/4)*32 + row%32)*4 + d%4.  Stage 3 consumes exactly this order. */
 int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn,
                          const void* k, int64_t k_sb, int64_t k_sh, int64_t k_sn,
@@ -97,7 +97,7 @@ int aa_stage1_anchor_fwd(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn
 /* ---- stage 2: difference-aware stripe identification -------------------------------------- */
 
 /* Mean-pools raw queries and anchors over block_size rows, rounding to the 16-bit type
- * (get_mask_test.py:75-84): qbar [B,Hq,N/block_size,128], abar [B,Hq,N/block_size], both of the tensors' 16-bit type.
+ * (get_mask_test.py:75-84): qbar [B,Hq,N/block_size,head_dim], abar [B,Hq,N/block_size], both of the tensors' 16-bit type.
  * Sums run in float32 in ascending row order. */
 int aa_pool_q_anchor(const void* q, int64_t q_sb, int64_t q_sh, int64_t q_sn, const float* M,
                      void* qbar, void* abar,

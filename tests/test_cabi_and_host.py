@@ -45,7 +45,9 @@ def test_host_geometry_helpers():
     ws = lib.aa_workspace_bytes(1, 32, 131072, 128, 128, 16)
     acc = 32 * 131072 * 128 * 4
     assert acc < ws < acc + 2**30
-    assert lib.aa_workspace_bytes(1, 32, 131072, 64, 128, 16) == 0  # head_dim 64 not supported
+    ws64 = lib.aa_workspace_bytes(1, 32, 131072, 64, 128, 16)  # head_dim 64: half the accumulator state and pooled queries
+    assert ws - ws64 == acc // 2 + 32 * 1024 * 64 * 2
+    assert lib.aa_workspace_bytes(1, 32, 131072, 96, 128, 16) == 0  # other head dimensions are not supported
 
 
 def test_error_codes_without_touching_the_gpu():
@@ -57,7 +59,7 @@ def test_error_codes_without_touching_the_gpu():
     dense = lambda q, nq, nkv, n, d, qs=s: lib.aa_dense_causal_fwd(q, *qs, p, *s, p, *s, p, *s, 1, nq, nkv, n, d, 0.1, 0, None)
     assert dense(None, 2, 2, 2048, 128) == 1 and b"q is NULL" in lib.aa_last_error()
     assert dense(p, 3, 2, 2048, 128) == 1 and b"divide" in lib.aa_last_error()
-    assert dense(p, 2, 2, 2048, 64) == 2 and b"head_dim" in lib.aa_last_error()
+    assert dense(p, 2, 2, 2048, 96) == 2 and b"head_dim" in lib.aa_last_error()  # 128 and 64 are the supported sizes
     assert dense(p, 2, 2, 2000, 128) == 2
     assert dense(p + 2, 2, 2, 2048, 128) == 3 and b"aligned" in lib.aa_last_error()
     assert dense(p, 2, 2, 2048, 128, qs=(s[0], s[1], 132)) == 3
@@ -74,7 +76,7 @@ def test_error_codes_without_touching_the_gpu():
     assert rc == 1 and b"scale_mode" in lib.aa_last_error()
     rc = lib.aa_stage1_anchor_fwd(p, *s, p, *s, p, *s, p, p, p, 1, 2, 2, 2048, 128, 128, 16, 0.1, 0, 5, None)
     assert rc == 1 and b"dtype" in lib.aa_last_error()
-    assert lib.aa_version() == 2
+    assert lib.aa_version() == 3
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -226,4 +228,6 @@ def test_bench_cli_contract_without_a_gpu():
     assert f2 == 32 * 2 * 16 * 128 * sum(bb * 2048 - 256 for bb in range(1, 64))
     assert f3 == 4 * 128 * 2048 * 855140
     assert abs((f1 + f2 + f3) / 1e12 - 8.10) < 0.01
-    assert set(bench.WORKLOADS) == {"config0_llama8b_4k", "config1_llama8b_32k", "config2_llama8b_128k", "config3_qwen7b_64k"}
+    assert set(bench.WORKLOADS) == {"config0_llama8b_4k", "config1_llama8b_32k", "config2_llama8b_128k", "config3_qwen7b_64k",
+                                    "llama1b_128k_headdim64"}
+    assert bench.workload_head_dim("config2_llama8b_128k") == 128 and bench.workload_head_dim("llama1b_128k_headdim64") == 64

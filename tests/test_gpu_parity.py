@@ -61,7 +61,7 @@ def _packed_lists(hip, coords, counts, N, step=STEP, bs=BS):
     return out, counts
 
 
-def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP, bs=BS, dtype="bf16"):
+def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused, step=STEP, bs=BS, dtype="bf16", sm=SM):
     """Sets equal except excused keys (flip distance < BAND); returns number of excused keys."""
     S = bs * step
     B, Hq = got_counts.shape[:2]
@@ -83,7 +83,7 @@ def _assert_index_parity(ao, got, got_counts, want, Q, K, M, theta, max_excused,
                     abar, mean = ao.pooled_anchors(M[b, h], bs, dtype)
                 rows = slice(bb * step, (bb + 1) * step)
                 for j in sym:
-                    d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], SM, theta, dtype)
+                    d = ao.stage2_flip_distance(qbar[rows], abar[rows], mean[rows], K[b, h // group, j], sm, theta, dtype)
                     assert d < BAND, f"key {j} (b={b},h={h},bb={bb}) differs and is {d:.4g} from any decision flip"
                     excused += 1
     assert excused <= max_excused, f"{excused} near-threshold disagreements"
@@ -559,7 +559,7 @@ def test_theta_sweep_tooling(mods):
     assert wide[1]["recall@0.01"] >= wide[0]["recall@0.01"]
 
 
-def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16"):
+def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16", sm=SM):
     """Stages 1 and 3 on sampled (head, row) pairs, recomputed in float64 on the host (P rounded to bf16 as the
     kernels do) from the kernel's own index lists; returns the per-row max errors."""
     N = q.shape[2]
@@ -572,7 +572,7 @@ def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16
         K1 = k[0, kv, keys1].double().cpu().numpy()
         V1 = v[0, kv, keys1].double().cpu().numpy()
         qrow = q[0, h, r].float().cpu().numpy()
-        q1 = ao.q1_scale_chain(qrow[None], SM, dtype=dtype)[0].astype(np.float64)
+        q1 = ao.q1_scale_chain(qrow[None], sm, dtype=dtype)[0].astype(np.float64)
         s1 = K1 @ q1
         m1 = s1.max()
         p1 = np.exp2(s1 - m1)
@@ -581,7 +581,7 @@ def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16
         assert abs(float(M[0, h, r]) - m1) < 3e-4
         assert abs(float(L[0, h, r]) - l1) / l1 < 1e-3
         lst = index_list(h, bb)
-        q3 = ao.q3_scale_chain(qrow[None], SM, dtype=dtype)[0].astype(np.float64)
+        q3 = ao.q3_scale_chain(qrow[None], sm, dtype=dtype)[0].astype(np.float64)
         if lst.size:
             K3 = k[0, kv, lst].double().cpu().numpy()
             V3 = v[0, kv, lst].double().cpu().numpy()

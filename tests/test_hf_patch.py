@@ -6,11 +6,11 @@ import pytest
 import torch
 
 
-def _tiny(n_layers=2, **kw):
+def _tiny(n_layers=2, head_dim=128, **kw):
     from transformers import LlamaConfig, LlamaForCausalLM
     torch.manual_seed(0)
-    cfg = LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=n_layers, num_attention_heads=4,
-                      num_key_value_heads=2, head_dim=128, vocab_size=1000, max_position_embeddings=16384,
+    cfg = LlamaConfig(hidden_size=4 * head_dim, intermediate_size=1024, num_hidden_layers=n_layers, num_attention_heads=4,
+                      num_key_value_heads=2, head_dim=head_dim, vocab_size=1000, max_position_embeddings=16384,
                       rope_theta=5e5, **kw)
     return LlamaForCausalLM(cfg).eval()
 
@@ -195,12 +195,14 @@ def test_plug_sparse_branch_is_the_operator_plus_dense_tail(n_tokens, monkeypatc
 
 
 @pytest.mark.gpu
-def test_patched_model_equals_dense_model_when_the_window_covers_everything():
+@pytest.mark.parametrize("head_dim", [128, 64])
+def test_patched_model_equals_dense_model_when_the_window_covers_everything(head_dim):
     """theta -> -inf selects nothing; with two big blocks the stage-1 window [0,S) U [bb*S, r] is the whole causal
-    prefix, so a patched model must reproduce the dense (SDPA) model's logits - prefill with a ragged tail."""
+    prefix, so a patched model must reproduce the dense (SDPA) model's logits - prefill with a ragged tail.  Both head
+    dimensions the kernels are built for (64: the Llama-3.2-1B / Qwen2.5-0.5B class of models)."""
     from anchor_attn import patch_model
-    ref = _tiny().to(torch.bfloat16).cuda()
-    m = _tiny().to(torch.bfloat16).cuda()
+    ref = _tiny(head_dim=head_dim).to(torch.bfloat16).cuda()
+    m = _tiny(head_dim=head_dim).to(torch.bfloat16).cuda()
     m.load_state_dict(ref.state_dict())
     patch_model(m, "anchor_attn", {"theta": -1e4})
     x = torch.randint(0, 1000, (1, 2 * 2048 + 77), device="cuda")

@@ -252,14 +252,15 @@ def test_stage3_multiplicity_closed_form(small):
     assert (sel & wmask).any()
 
 
-def _closed_form_check(bs, step, n_bb, dtype):
+def _closed_form_check(bs, step, n_bb, dtype, head_dim=D):
     """The whole operator against an independent route: float64 window/selection masks and the multiplicity closed form
     for the output, torch casts to the 16-bit type and float64 dots for the selection - none of it shares code with the
     oracle's tile loops."""
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float16
     S_ = bs * step
     N = n_bb * S_
-    q, k, v, _ = make_qkv(N, 2, 1, n_stripes=max(8, N // 64), seed=300 + bs, dtype=tdt)
+    sm = SM if head_dim == D else 1.0 / np.sqrt(head_dim)
+    q, k, v, _ = make_qkv(N, 2, 1, head_dim=head_dim, n_stripes=max(8, N // 64), seed=300 + bs, dtype=tdt)
     Q, K, V = _np(q, k, v)
     theta = 12.0
     res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta, dtype=dtype)
@@ -273,12 +274,12 @@ def _closed_form_check(bs, step, n_bb, dtype):
     for h in range(2):
         # ---- selection, independently
         qt = torch.from_numpy(Q[0, h])
-        qbar = (qt.view(N // bs, bs, D).double().sum(1) / bs).float().to(tdt)
-        s1 = ao.q1_scale_chain(Q[0, h], SM, dtype=dtype).astype(np.float64) @ k64.T
+        qbar = (qt.view(N // bs, bs, head_dim).double().sum(1) / bs).float().to(tdt)
+        s1 = ao.q1_scale_chain(Q[0, h], sm, dtype=dtype).astype(np.float64) @ k64.T
         m_rows = np.where(wmask, s1, -np.inf).max(1)                       # the anchors are the windowed row maxima
         np.testing.assert_allclose(res.M[0, h], m_rows, atol=2e-4)
         abar = (torch.from_numpy(res.M[0, h]).view(N // bs, bs).double().sum(1) / bs).float().to(tdt)
-        sc = ((qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (SM * ao.LOG2E)).float().to(tdt)
+        sc = ((qbar.double() @ torch.from_numpy(K[0, 0]).double().T) * (sm * ao.LOG2E)).float().to(tdt)
         hit = ((sc.float() + diff) >= abar.float()[:, None]).view(n_bb, step, N).any(1)
         sel = np.zeros((N, N), bool)
         for bb in range(n_bb):
@@ -289,7 +290,7 @@ def _closed_form_check(bs, step, n_bb, dtype):
             assert len(set(want.tolist()) ^ set(got.tolist())) <= 2          # float64 vs float32 dots at a boundary
             sel[bb * S_:(bb + 1) * S_, got] = True
         # ---- output: multiplicity closed form
-        s3 = ao.q3_scale_chain(Q[0, h], SM, dtype=dtype).astype(np.float64) @ k64.T
+        s3 = ao.q3_scale_chain(Q[0, h], sm, dtype=dtype).astype(np.float64) @ k64.T
         a = np.where(wmask, s1, -np.inf)
         b = np.where(sel, s3, -np.inf)
         mx = np.maximum(a.max(1), b.max(1))
@@ -304,6 +305,14 @@ def test_other_block_sizes_by_independent_closed_form(bs, step, n_bb):
     """block_size is a parameter of all three stages (pooling width, candidate range [bs, bb*S - bs), big block
     S = bs*step, window [0,S) U [bb*S, r]): every block size the reference's assert admits."""
     _closed_form_check(bs, step, n_bb, "bf16")
+
+
+@pytest.mark.parametrize("bs,step,n_bb,dtype", [(128, 16, 3, "bf16"), (64, 16, 4, "bf16"), (128, 16, 2, "fp16")])
+def test_head_dim_64_by_independent_closed_form(bs, step, n_bb, dtype):
+    """The reference's kernels take the head dimension from the tensors (anchor_attn_v4.py:263, anchor_step_1_2_v2.py:21);
+    the default softmax scale is then 1/sqrt(64) = 0.125, which both scale chains represent exactly."""
+    res = _closed_form_check(bs, step, n_bb, dtype, head_dim=64)
+    assert res.out.shape[-1] == 64
 
 
 # ---------------------------------------------------------------- fp16 tensors
