@@ -42,7 +42,7 @@
 namespace aa {
 
 constexpr int kBN = 64;        // keys per LDS tile
-constexpr int kRowBytes = 256;   // one K/V row in LDS (128 bf16, unpadded, chunks swizzled)
+constexpr int kRowBytes = 256;   // pitch of a K/V row in LDS (128 16-bit elements, unpadded, chunks swizzled; head dimension 64 fills half)
 constexpr int kTileBytes = kBN * kRowBytes;
 constexpr int kDist = 4;         // MFMA operands are fetched from LDS this many MFMAs ahead of their use
 constexpr int kIdxWin = 1024;    // selected-key indices held in LDS at a time (16 tiles)
