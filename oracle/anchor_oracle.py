@@ -24,6 +24,8 @@ bit for bit against the Triton toolchain itself: tests/triton_promotion_probe.py
 forms of the reference's expression as micro-kernels of its own, and its outputs on an MI355X are
 the fixture tests/golden/triton_scale_chain_probe.npz (made with Triton 3.6.0; the reference's
 requirements.txt pins 3.2.0, which is not installed here).  ``stage1_scale_mode`` remains a switch.
+Nothing here depends on the head dimension (the reference's kernels take ``D`` from the tensors); besides 128 the
+pins run at 64 (tests/test_oracle_pins.py::test_head_dim_64_by_independent_closed_form).
 
 Conventions: ``Q`` is ``[B, Hq, N, D]``, ``K``/``V`` are ``[B, Hkv, N, D]`` with ``Hkv | Hq``
 (query head ``h`` reads KV head ``h // (Hq // Hkv)``, the order ``repeat_kv`` produces);
