@@ -231,3 +231,30 @@ def test_bench_cli_contract_without_a_gpu():
     assert set(bench.WORKLOADS) == {"config0_llama8b_4k", "config1_llama8b_32k", "config2_llama8b_128k", "config3_qwen7b_64k",
                                     "llama1b_128k_headdim64"}
     assert bench.workload_head_dim("config2_llama8b_128k") == 128 and bench.workload_head_dim("llama1b_128k_headdim64") == 64
+
+
+def test_get_mask_block_restatement_agrees_with_the_oracle():
+    """``get_mask_block`` (the framework-tensor restatement of stage 2 that the reference keeps next to its kernel,
+    get_mask_test.py:162-232) against the oracle's stage 2 on the oracle's own anchors: the same candidate range
+    [bs, i*S - bs), ascending lists in the reference's buffer layout, zero for big block 0; the two differ only by the
+    kernels' rounding points, i.e. by keys within rounding of the threshold."""
+    from anchor_attn.src.ops.get_mask_test import get_mask_block
+    from oracle import anchor_oracle as ao
+    n, bs, step = 3 * 2048, 128, 16
+    q, k, v, _ = make_qkv(n, 2, 1, n_stripes=96, seed=5)
+    res = ao.anchor_attn_reference(q.float().numpy(), k.float().numpy(), v.float().numpy(), difference=12.0)
+    sm = 128 ** -0.5
+    coords, counts, ratio = get_mask_block(q.float(), k.repeat_interleave(2, 1).float(), torch.from_numpy(res.M), bs, bs, step,
+                                           12.0 * ao.LOG2E, 1, 2, n, 128, sm * ao.LOG2E, "cpu", True)
+    assert coords.shape == (1, 2, 3, n) and coords.dtype == torch.int32 and counts.shape == (1, 2, 3, 1)
+    assert int(counts[0, :, 0].sum()) == 0
+    total = 0
+    for h in range(2):
+        for bb in range(3):
+            c = int(counts[0, h, bb, 0])
+            got = coords[0, h, bb, :c].numpy()
+            assert np.all(np.diff(got) > 0) and (c == 0 or (got[0] >= bs and got[-1] < bb * bs * step - bs))
+            assert int(coords[0, h, bb, c:].abs().sum()) == 0
+            assert len(set(got.tolist()) ^ set(res.coords[0][h][bb].tolist())) <= 2
+            total += c
+    assert total > 0 and abs(ratio - total / (2 * ((2048 - 256) + (4096 - 256)))) < 1e-12
