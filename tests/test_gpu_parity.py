@@ -15,6 +15,25 @@ LOG2E = 1.44269504
 MAX_ERR, MEAN_ERR, BAND = 2e-2, 2e-3, 1e-3
 
 
+def _assert_outputs_close(got, want, dtype="bf16", what=""):
+    """The operator's output bar: max |err| <= 2e-2 and mean |err| <= 2e-3.  One exception, counted and kept rare: where
+    the output's own grid is coarser than the bar - a bf16 value of magnitude 4 or more has a spacing of 2^-5 = 0.03125 -
+    two correct roundings of nearly equal sums can land on neighbouring grid points, so a difference of exactly one
+    grid step is accepted there (at most ten elements per million)."""
+    got = np.asarray(got, dtype=np.float32)
+    want = np.asarray(want, dtype=np.float32)
+    err = np.abs(got - want)
+    assert err.mean() <= MEAN_ERR, (what, float(err.mean()))
+    over = err > MAX_ERR
+    if over.any():
+        mant_bits = 7 if dtype == "bf16" else 10
+        step = np.exp2(np.floor(np.log2(np.maximum(np.abs(want[over]), np.abs(got[over])))) - mant_bits)
+        assert np.all(err[over] <= step * 1.0001), (what, float(err.max()))
+        assert over.sum() <= 1 + 1e-5 * err.size, (what, int(over.sum()), err.size)
+    return err
+
+
+
 def _np(*ts):
     return [t.float().cpu().numpy() for t in ts]
 
@@ -171,28 +190,30 @@ def test_stage3_matches_oracle_given_same_state(mods, llama_small):
     got_lists, got_counts = _packed_lists(hip, coords, counts, N)
     want = ao.stage3_sparse(Q, K, V, got_lists, got_counts, M.cpu().numpy(), L.cpu().numpy(),
                             st.acc_rows(Acc).cpu().numpy(), SM)
-    err = np.abs(out.float().cpu().numpy() - want)
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    _assert_outputs_close(out.float().cpu().numpy(), want)
 
 
 # ------------------------------------------------------------------------------------ whole operator
 def _end_to_end(mods, q, k, v, theta, max_excused=6, step=STEP, bs=BS):
+    """The whole operator against the oracle on the same inputs (any supported head dimension, grouping, block size,
+    step, element type): anchors, index sets, output, ratio."""
     hip, v4, st, ao = mods
     Q, K, V = _np(q, k, v)
     dtype = "fp16" if q.dtype == torch.float16 else "bf16"
+    d = q.shape[-1]
+    sm = 1.0 / math.sqrt(d)
     res = ao.anchor_attn_reference(Q, K, V, block_size=bs, step=step, difference=theta, dtype=dtype)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     out, ratio = v4.anchor_attn(qd, kd, vd, block_size=bs, step=step, difference=theta)
     B, H, N, _ = q.shape
     # stage outputs for index parity come from the staged entry points on the same inputs
-    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, bs, step, B, H, N, D, SM)
+    L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, bs, step, B, H, N, d, sm)
     np.testing.assert_allclose(M.cpu().numpy(), res.M, atol=3e-4)
-    coords, counts = st.select_stripes_packed(qd, kd, M, bs, step, theta * LOG2E, B, H, N, D, SM)
+    coords, counts = st.select_stripes_packed(qd, kd, M, bs, step, theta * LOG2E, B, H, N, d, sm)
     got, got_counts = _packed_lists(hip, coords, counts, N, step, bs)
-    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step, bs, dtype)
+    _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, max_excused, step, bs, dtype, sm=sm)
     assert out.dtype == q.dtype
-    err = np.abs(out.float().cpu().numpy() - res.out)
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
+    _assert_outputs_close(out.float().cpu().numpy(), res.out, dtype)
     want_ratio = got_counts.sum() / ((B * H * N * N / (bs * step)) // 2)
     assert abs(float(ratio) - want_ratio) < 1e-6
     return res, out
@@ -208,6 +229,44 @@ def test_anchor_attn_end_to_end_qwen_grouping(mods):
     """GQA 7:1 (not a power of two), RoPE base 1e6, 4 big blocks."""
     q, k, v, _ = _case(4 * S, 7, 1, 128, seed=33, rope_base=1e6)
     _end_to_end(mods, q, k, v, 12.0)
+
+
+def _random_configurations(n, seed):
+    """Seeded draws from the supported parameter space: head dimension, element type, block size, step, grouping,
+    number of big blocks (kept small enough for the CPU oracle), threshold, batch."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        d = int(rng.choice([128, 64]))
+        bs = int(rng.choice([16, 32, 64, 128, 256]))
+        step = int(rng.choice([16, 32]))
+        big = bs * step
+        n_bb = int(rng.integers(1, max(2, min(6, 12288 // big) + 1)))
+        hkv = int(rng.choice([1, 2, 3]))
+        group = int(rng.choice([1, 2, 4, 7]))
+        while hkv * group * (n_bb * big) ** 2 > 6e8 and (n_bb > 1 or group > 1):  # keeps the CPU oracle within ~15 s per case
+            if n_bb > 1:
+                n_bb -= 1
+            else:
+                group = {7: 4, 4: 2, 2: 1}[group]
+        theta = float(rng.choice([9.0, 11.5, 12.0, 13.0, 14.5]))
+        dtype = torch.float16 if rng.random() < 0.3 else torch.bfloat16
+        batch = 2 if rng.random() < 0.2 else 1
+        cases.append((i, d, bs, step, n_bb, hkv, group, theta, dtype, batch, float(rng.choice([5e5, 1e6]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_configurations(24, 20240917), ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c[:10]))
+def test_seeded_sweep_of_valid_configurations(mods, case):
+    """The parameters the interface admits, drawn together rather than one at a time: every draw must meet the
+    operator's parity bars against the oracle (anchors, index sets up to the flip band, outputs, ratio)."""
+    from anchor_attn.synthetic import make_qkv
+    i, d, bs, step, n_bb, hkv, group, theta, dtype, batch, base = case
+    n = n_bb * bs * step
+    parts = [make_qkv(n, hkv * group, hkv, head_dim=d, rope_base=base, n_stripes=max(4, n // 96), seed=7000 + 10 * i + b, dtype=dtype)[:3]
+             for b in range(batch)]
+    q, k, v = (torch.cat(t, 0) for t in zip(*parts))
+    _end_to_end(mods, q, k, v, theta, max_excused=12, step=step, bs=bs)
 
 
 def test_anchor_attn_config0_shape(mods):
@@ -508,8 +567,7 @@ def test_intended_geometry_mode(mods):
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     res = ao.anchor_attn_reference(Q, K, V, difference=12.0, strict_reference=False)
     out, ratio = v4.anchor_attn(qd, kd, vd, difference=12.0, strict_reference=False)
-    err = np.abs(out.float().cpu().numpy() - res.out)
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    _assert_outputs_close(out.float().cpu().numpy(), res.out)
     B, H, N, _ = q.shape
     L, M, Acc = st.anchor_attn_step_1(qd, kd, vd, 1, 1, BS, STEP, B, H, N, D, SM)
     coords, counts = st.select_stripes_packed(qd, kd, M, BS, STEP, 12.0 * LOG2E, B, H, N, D, SM, geometry=hip.AA_GEOMETRY_INTENDED)
@@ -592,8 +650,7 @@ def _check_sampled_rows(ao, q, k, v, M, L, out, index_list, samples, dtype="bf16
             den = l1 * np.exp2(m1 - m) + p3.sum()
         else:
             num, den = a1, l1
-        err = np.abs(out[0, h, r].double().cpu().numpy() - num / den)
-        assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (h, r, err.max(), err.mean())
+        err = _assert_outputs_close(out[0, h, r].float().cpu().numpy(), num / den, dtype, what=(h, r))
         errs.append(err.max())
     return errs
 
@@ -776,8 +833,7 @@ def test_gpu_matches_committed_fixture(mods):
     rows = torch.from_numpy(fx.ROWS).cuda()
     np.testing.assert_allclose(M[0][:, rows].cpu().numpy(), want["M"], atol=3e-4)
     np.testing.assert_allclose(L[0][:, rows].cpu().numpy(), want["L"], rtol=1e-3)
-    err = np.abs(out[0][:, rows].float().cpu().numpy() - want["out"])
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    _assert_outputs_close(out[0][:, rows].float().cpu().numpy(), want["out"])
     assert abs(float(ratio) - float(want["ratio"])) < 1e-4
 
 

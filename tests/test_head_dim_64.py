@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from test_gpu_parity import BAND, LOG2E, MAX_ERR, MEAN_ERR, _assert_index_parity, _np, _packed_lists, mods  # noqa: F401
+from test_gpu_parity import LOG2E, _assert_index_parity, _assert_outputs_close, _np, _packed_lists, mods  # noqa: F401
 
 pytestmark = pytest.mark.gpu
 
@@ -50,8 +50,7 @@ def test_end_to_end(mods, n_bb, hq, hkv, bs, step, theta, seed, base, dtype):
     got, got_counts = _packed_lists(hip, coords, counts, N, step, bs)
     _assert_index_parity(ao, got, got_counts, res.coords, Q, K, res.M, theta, 8, step, bs, name, sm=SM)
     assert (res.counts.sum() > 0 or n_bb == 1) and out.dtype == dtype
-    err = np.abs(out.float().cpu().numpy() - res.out)
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR, (err.max(), err.mean())
+    _assert_outputs_close(out.float().cpu().numpy(), res.out, name)
     assert abs(float(ratio) - got_counts.sum() / ((B * H * N * N / (bs * step)) // 2)) < 1e-6
     # the one-call entry point (pooling fused into stage 1 for block sizes up to 128) against the staged ones
     staged, ratio2 = v4.anchor_attn_without_anchor(qd, kd, vd, block_size=bs, step=step, difference=theta)
@@ -91,8 +90,7 @@ def test_stages_pooling_and_dense_baseline(mods):
     out = v4._stage3(qd, kd, vd, coords, counts, L, M, Acc, SM, bs, step)
     lists, cnts = _packed_lists(hip, coords, counts, N)
     want = ao.stage3_sparse(Q, K, V, lists, cnts, M.cpu().numpy(), L.cpu().numpy(), st.acc_rows(Acc).cpu().numpy(), SM)
-    err = np.abs(out.float().cpu().numpy() - want)
-    assert err.max() <= MAX_ERR and err.mean() <= MEAN_ERR
+    _assert_outputs_close(out.float().cpu().numpy(), want)
     dense = v4.dense_causal_attention(qd, kd, vd)
     ref = torch.nn.functional.scaled_dot_product_attention(
         q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
