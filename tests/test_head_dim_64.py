@@ -31,6 +31,8 @@ def _case64(n_ctx, hq, hkv, n_stripes, seed, **kw):
     (1, 4, 2, 128, 16, 12.0, 607, 5e5, torch.bfloat16),   # a single big block: nothing to select
     (6, 2, 1, 16, 16, 12.0, 608, 5e5, torch.bfloat16),    # block size 16: eight pooled rows per 128-row work-group
     (3, 2, 2, 32, 32, 12.0, 609, 5e5, torch.bfloat16),    # block size 32, step 32
+    (3, 2, 1, 128, 16, 1e4, 610, 5e5, torch.bfloat16),    # every candidate selected: lists of 1792 and 3840 entries (the
+                                                          # sparse kernel refills its 1024-entry index window)
 ])
 def test_end_to_end(mods, n_bb, hq, hkv, bs, step, theta, seed, base, dtype):
     hip, v4, st, ao = mods
