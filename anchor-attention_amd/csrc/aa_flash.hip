@@ -62,6 +62,9 @@ enum FlashMode : int { kAnchor = 0, kSparse = 1, kDense = 2 };
 #ifndef AA_ABLATE
 #define AA_ABLATE 0
 #endif
+#ifndef AA_SPARSE_CHAIN
+#define AA_SPARSE_CHAIN 1  // 0: every query block of a stage-3 work-group requests its own first tile, queries and state
+#endif
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -70,13 +73,10 @@ typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
 
 template <bool WITH_IDX>
 struct FlashSmem {
-  union {
-    struct {
-      char k[2][kTileBytes];
-      char v[2][kTileBytes];
-    } t;
-    uint16_t os[4][32 * 136];  // epilogue staging (row stride D + 8 elements), reuses the tile space
-  };
+  struct {
+    char k[2][kTileBytes];
+    char v[2][kTileBytes];
+  } t;  // (the epilogue stages the output in the tile space)
   int32_t idx[WITH_IDX ? kIdxWin : 4];  // sparse mode: window of the big block's index list
 };
 
@@ -153,7 +153,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   constexpr int kDB = D / 32;       // 32-column blocks of the head dimension: accumulators of O^T
   constexpr int kNS = 2 * kKS;      // S^T slots of a 64-key tile
   constexpr int kNV = 4 * kDB;      // O^T slots of a 64-key tile (two 16-key steps per 32-key block)
-  constexpr int kOsStride = D + 8;  // 16-bit elements per output-staging row in LDS
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -206,6 +205,55 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
   const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
 
+  // ---- sparse mode: what the query blocks of a work-group share, and what they hand to each other -------
+  // All blocks lie in one big block of one head, so they walk the same index list and gather the same tiles.  When the
+  // list fits the LDS window, the blocks are chained: the last tile of a block brings the list's first tile into the idle
+  // buffer for the next block, whose queries and statistics are requested before the output of the block is staged and
+  // whose accumulator state is requested as soon as the staging has emptied the accumulator registers - so the next
+  // block starts its first product without a round trip to memory of its own.
+  int cnt = 0, cap = 0, sparse_tiles = 0;
+  const int32_t* cbase = nullptr;
+  if (MODE == kSparse) {
+    cap = max(bb * S - 2 * p.block_size, 0);  // capacity of the big block's list (a multiple of 4)
+    // (counts and indices come from device memory the caller filled: a count beyond the capacity or an index beyond
+    // the context is clamped rather than followed out of bounds)
+    cnt = max(0, min(p.counts[bh * (p.n_ctx / S) + bb], cap));
+    cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
+    sparse_tiles = (cnt + kBN - 1) / kBN;
+    if (AA_ABLATE == 4 || AA_ABLATE == 7) sparse_tiles = 0;
+    if (AA_ABLATE == 6) sparse_tiles = min(sparse_tiles, 2);
+  }
+  const bool list_chains = MODE == kSparse && AA_SPARSE_CHAIN && sparse_tiles > 0 && sparse_tiles <= kIdxWin / kBN;
+  int cur = 0;             // (sparse) LDS buffer of the next tile to be computed
+  bool chained = false;    // (sparse) this block's first tile and state were requested by the previous block
+  bool have_queries = false;  // (sparse) so were its queries and statistics
+  u32x4 qraw[kKS];
+  float m_in = 0.f, l_in = 0.f;
+  floatx16 acc[kDB];
+  // (sparse) queries and soft-max statistics of the block whose lane row is `row`
+  auto request_queries = [&](const int row) __attribute__((always_inline)) {
+    const uint16_t* qr = qp + (int64_t)row * p.q_sn + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qr + 16 * ks);
+    m_in = p.M[bh * p.n_ctx + row];
+    l_in = half == 0 ? p.L[bh * p.n_ctx + row] : 0.f;  // the two halves are summed at the end
+  };
+  // (sparse) the accumulator state of that block.  (The accumulator state and the output are touched once each: they
+  // are written and read with the non-temporal hint, so that they do not push K/V rows, which many work-groups share,
+  // out of the L2.)
+  auto request_state = [&](const int row) __attribute__((always_inline)) {
+    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + row / 32) * (4 * kDB)) * 256 + lane * 4;
+#pragma unroll
+    for (int db = 0; db < kDB; ++db)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        floatx4 t = {0.f, 0.f, 0.f, 0.f};
+        if (AA_ABLATE != 5 && AA_ABLATE != 7) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256));
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
+      }
+  };
+
   for (int qb = 0; qb < nq; ++qb) {
   const int R0 = (qunit * nq + qb) * BM;
   const int wr0 = R0 + wave * 32;
@@ -215,35 +263,21 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   // They depend on nothing, whereas the first K/V tile needs the index list, which needs its own round trip to
   // memory.  The 64 KB of accumulator state follow the first tile's loads (further down) and are not waited for
   // before the first scores are computed.
-  u32x4 qraw[kKS];
   float m_run, l_run;
-  floatx16 acc[kDB];
   const uint16_t* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
-  if (MODE == kSparse) {
-#pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) qraw[ks] = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
-    m_run = p.M[bh * p.n_ctx + my_row];
-    l_run = half == 0 ? p.L[bh * p.n_ctx + my_row] : 0.f;  // the two halves are summed at the end
-  }
+  if (MODE == kSparse && !have_queries) request_queries(my_row);
+  const bool feeds_next = list_chains && qb + 1 < nq;  // the next block takes its first tile from this one
 
   // ---- tile schedule -------------------------------------------------------------------------
   const bool pool = MODE == kAnchor && p.qbar_out != nullptr;
-  int n_tiles, n_init = 0, cnt = 0, cap = 0;
-  const int32_t* cbase = nullptr;
+  int n_tiles, n_init = 0;
   if (MODE == kAnchor) {
     n_init = min(S, R0 + BM) / kBN;
     n_tiles = n_init + (bb >= 1 ? (R0 + BM - bb * S) / kBN : 0);
   } else if (MODE == kDense) {
     n_tiles = (R0 + BM) / kBN;
   } else {
-    cap = max(bb * S - 2 * p.block_size, 0);  // capacity of the big block's list (a multiple of 4)
-    // (counts and indices come from device memory the caller filled: a count beyond the capacity or an index beyond
-    // the context is clamped rather than followed out of bounds)
-    cnt = max(0, min(p.counts[bh * (p.n_ctx / S) + bb], cap));
-    cbase = p.coords + bh * p.coords_per_head + coords_tri(bb, S, p.block_size);
-    n_tiles = (cnt + kBN - 1) / kBN;
-    if (AA_ABLATE == 4 || AA_ABLATE == 7) n_tiles = 0;
-    if (AA_ABLATE == 6) n_tiles = min(n_tiles, 2);
+    n_tiles = sparse_tiles;
   }
   // first key (anchor, dense) or first list position (sparse) of tile i
 #define AA_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
@@ -284,27 +318,15 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const char* qblock = reinterpret_cast<const char*>(qp + (int64_t)R0 * p.q_sn);
   const uint32_t q_row_bytes = (uint32_t)p.q_sn * 2u;
   const uint32_t q_voff = (uint32_t)(tid >> 4) * q_row_bytes + (uint32_t)((tid & 15) & (D / 8 - 1)) * 16u;
-  if (n_tiles > 0) {
+  if (n_tiles > 0 && !chained) {
+    const uint32_t first = MODE == kSparse ? (uint32_t)cur * kTileBytes : 0u;
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0, lds_v0,
-                           k_voff, v_voff);
+      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0 + first,
+                           lds_v0 + first, k_voff, v_voff);
   }
-  if (MODE == kSparse) {
-    // the accumulator state: the youngest loads in flight, first needed by the first P.V product.  (The accumulator
-    // state and the output are touched once each: they are written and read with the non-temporal hint, so that they
-    // do not push K/V rows, which many work-groups share, out of the L2.)
-    const float* af = p.acc_frag + ((bh * (p.n_ctx / 32) + my_row / 32) * (4 * kDB)) * 256 + lane * 4;
-#pragma unroll
-    for (int db = 0; db < kDB; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        floatx4 t = {0.f, 0.f, 0.f, 0.f};
-        if (AA_ABLATE != 5 && AA_ABLATE != 7) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(af + (db * 4 + rg) * 256));
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[db][rg * 4 + c] = t[c];
-      }
-  }
+  // the accumulator state: the youngest loads in flight, first needed by the first P.V product
+  if (MODE == kSparse && !chained) request_state(my_row);
 
   // ---- queries: B operand, pre-scaled into the exp2 domain -----------------------------------
   vec8 qreg[kKS];
@@ -326,6 +348,9 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     for (int db = 0; db < kDB; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+  } else {
+    m_run = m_in;
+    l_run = l_in;
   }
 
   // m_ref is what the score accumulators are pre-loaded with (negated); it equals m_run except before
@@ -339,8 +364,13 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // Loads complete in order and the accumulator state was requested last, with 4 * kDB load instructions, so "at most
     // that many outstanding" means: everything requested before it - queries, statistics, tile 0 - has arrived.  The
     // state itself may still be on its way while the first scores are computed (the compiler waits where it is first used).
-    if (kDB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    // (A chained block has nothing to wait for here: its first tile landed before the previous block's last barrier, and
+    // the compiler waits for the queries where they are scaled.  The barrier is still needed - the tile about to be
+    // requested lands where the other waves staged their output.)
+    if (!chained) {
+      if (kDB == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    }
     lds_barrier();  // a barrier that does not wait for the loads still in flight
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // tile 0 has landed in LDS
@@ -349,18 +379,24 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 
   // per-lane LDS byte offsets.  K: row c32 (+32*kb), chunk 2*ks + half, swizzled with the row's low four bits.
   // (absolute LDS addresses into the current buffer; the 32-key half and the row steps are immediate offsets)
+  const uint32_t first_buf = MODE == kSparse ? (uint32_t)cur * kTileBytes : 0u;  // (sparse) where this block's first tile lies
+  // (sparse: formed per block from an opaque copy of the lane number - hoisted out of the loop over the work-group's
+  // blocks, the pieces of these addresses would occupy registers throughout the tile loop)
+  int lane_t = lane;
+  if (MODE == kSparse) asm volatile("" : "+v"(lane_t));
+  const int c32_t = lane_t & 31, half_t = lane_t >> 5;
   uint32_t k_rd[kKS];
 #pragma unroll
-  for (int ks = 0; ks < kKS; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
+  for (int ks = 0; ks < kKS; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + first_buf + c32_t * kRowBytes + (((2 * ks + half_t) ^ (c32_t & 15)) << 4);
   // transposing V read i: a group of 16 lanes covers 16 head-dim columns; lane points at row r0 = 4*half + (lane%16)/4
   // (+ multiples of 8, which leave r0 = row & 7 alone), bf16 columns 32*(i&3) + 16*((lane>>4)&1) + 4*(lane&3): chunk
   // 4*(i&3) + y0 with y0 < 4, swizzled with r0 << 1 -> one offset per value of i & 3
   uint32_t v_rd[kDB];
   {
-    const int r0 = 4 * half + ((lane & 15) >> 2);
-    const int y0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int r0 = 4 * half_t + ((lane_t & 15) >> 2);
+    const int y0 = 2 * ((lane_t >> 4) & 1) + ((lane_t & 3) >> 1);
 #pragma unroll
-    for (int m = 0; m < kDB; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
+    for (int m = 0; m < kDB; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + first_buf + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane_t & 1);
   }
 
 
@@ -418,11 +454,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   // the buffer's offset is part of every LDS instruction's immediate offset and the read addresses are loop-invariant.
   // Sparse mode, whose tile counts can be odd, keeps one copy of the tile (BUF = -1): the buffer is i & 1 and the read
   // addresses step back and forth between the two buffers.
-  int32_t buf_step = kTileBytes;
+  int32_t buf_step = (MODE == kSparse && cur) ? -kTileBytes : kTileBytes;
   auto run_tile = [&](auto buf_const, const int i) __attribute__((always_inline)) {
     constexpr int kBuf = decltype(buf_const)::value;
     constexpr uint32_t rd_off = kBuf > 0 ? kBuf * kTileBytes : 0;  // immediate part of the LDS read addresses
-    const int buf = kBuf >= 0 ? kBuf : (i & 1);
+    const int buf = kBuf >= 0 ? kBuf : cur;
     const int key0 = AA_TILE_KEY0(i);
     if (MODE == kSparse && i + 1 < n_tiles && ((i + 1) & (kIdxWin / kBN - 1)) == 0) {
       // tile i+1 opens the next window; everyone finished reading the old one before the last barrier
@@ -436,7 +472,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // unless the work-group also pools its queries: then the eight load slots of the last tile bring the work-group's
     // 128 raw query rows into the idle buffer instead, rows 0..63 where K tiles go and rows 64..127 where V tiles go,
     // chunks in place)
-    const int i_next = i + 1 < n_tiles ? i + 1 : i;
+    // (sparse, chained: the last tile of a block fetches the list's first tile, for the next block)
+    const int i_next = i + 1 < n_tiles ? i + 1 : (feeds_next ? 0 : i);
     const int key0_next = AA_TILE_KEY0(i_next);
     const bool fetch_queries = MODE == kAnchor && pool && i + 1 == n_tiles;  // wave-uniform
     // (selects, not branches: the eight slots stay straight-line code; the base address is scalar, and the vector offset
@@ -620,6 +657,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
 #pragma unroll
       for (int m = 0; m < kDB; ++m) v_rd[m] += buf_step;
       buf_step = -buf_step;
+      cur ^= 1;
     }
     if (AA_ABLATE != 9) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile i+1 has landed in LDS
     if (AA_ABLATE != 8 && AA_ABLATE != 9) __syncthreads();
@@ -701,8 +739,21 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
       }
     }
   } else {
-    // out = bf16(acc / l): stage the wave's [32][D] tile in LDS, then write whole rows
-    uint16_t* os = sm.os[wave];
+    // out = bf16(acc / l): the wave stages its [32][D] tile in LDS - 32 rows of the tile pitch, 16-byte chunks swizzled
+    // with the row like a K tile - and writes whole rows.  The staging area is private to the wave (only a wave-local wait
+    // lies between its writes and its reads) and lies in the tile buffer the loop consumed last, which every wave has
+    // finished reading (the tile's closing barrier): waves 0, 1 in its K half, waves 2, 3 in its V half.  In sparse mode
+    // the other buffer may already hold the next block's first tile.
+    const bool more = MODE == kSparse && qb + 1 < nq;
+    if (more) request_queries(my_row + BM);  // (the registers of this block's raw queries are long free)
+    char* ob = (MODE == kSparse ? (wave < 2 ? sm.t.k[cur ^ 1] : sm.t.v[cur ^ 1]) + (wave & 1) * 32 * kRowBytes
+                                : sm.t.k[0] + wave * 32 * kRowBytes);
+    constexpr int kChunkMask = D / 8 - 1;
+    // (the staging offsets are the same for every block of the work-group; computed from an opaque copy of the lane
+    // number they are formed here, a few instructions per block, instead of occupying registers throughout the tile loop)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int c32_e = lane_e & 31, half_e = lane_e >> 5;
     const float inv = 1.0f / l_tot;
 #pragma unroll
     for (int db = 0; db < kDB; ++db)
@@ -711,20 +762,22 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
         u32x2 w;
         w[0] = T::pack(acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv);
         w[1] = T::pack(acc[db][rg * 4 + 2] * inv, acc[db][rg * 4 + 3] * inv);
-        *reinterpret_cast<u32x2*>(&os[c32 * kOsStride + 32 * db + 8 * rg + 4 * half]) = w;
+        *reinterpret_cast<u32x2*>(ob + c32_e * kRowBytes + (((4 * db + rg) ^ (c32_e & kChunkMask)) << 4) + 8 * half_e) = w;
       }
-    __syncthreads();
+    // the accumulator registers are free: the next block's state can be on its way while this block's output leaves
+    if (more && list_chains) request_state(my_row + BM);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the wave's LDS writes are done (and stay above this line)
     uint16_t* op = p.out + b * p.o_sb + hq * p.o_sh;
     constexpr int kLanesPerRow = D / 8, kRowsPerStore = 64 / kLanesPerRow;  // a row is D/8 pieces of 16 bytes
 #pragma unroll
     for (int it = 0; it < 32 / kRowsPerStore; ++it) {
-      const int r = it * kRowsPerStore + lane / kLanesPerRow, c = lane % kLanesPerRow;
-      const u32x4 w = *reinterpret_cast<const u32x4*>(&os[r * kOsStride + 8 * c]);
+      const int r = it * kRowsPerStore + lane_e / kLanesPerRow, c = lane_e % kLanesPerRow;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(ob + r * kRowBytes + ((c ^ (r & kChunkMask)) << 4));
       __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c));
     }
+    chained = more && list_chains;
+    have_queries = more;
   }
-  // the staging rows just read lie where the next block's first tile is about to land
-  if (MODE == kSparse && qb + 1 < nq) __syncthreads();
   }  // query blocks of the work-group
 }
 
