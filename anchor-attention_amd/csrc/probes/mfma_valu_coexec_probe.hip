@@ -71,7 +71,8 @@ static void run_rate(const char* name) {
 #define VALU(x) asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(x) : "v"(c1), "v"(c2))
 
 // role: 0 idle, 1 MFMAs only (four independent accumulators), 2 vector only, 3 interleaved (1 MFMA + 6 vector),
-//       4 bursts (8 MFMAs, then 48 vector), 5 interleaved (1 MFMA + 3 vector)
+//       4 bursts (8 MFMAs, then 48 vector), 5 interleaved (1 MFMA + 3 vector),
+//       6 MFMAs only, one dependent chain (every MFMA accumulates onto the previous one's result), 7 two alternating chains
 template <int ROLE_LO, int ROLE_HI>
 __global__ void __launch_bounds__(512) coexec(int iters, float* out, float c1, float c2) {
   const int wave = threadIdx.x >> 6;
@@ -101,6 +102,10 @@ __global__ void __launch_bounds__(512) coexec(int iters, float* out, float c1, f
 #pragma unroll
       for (int j = 0; j < 8; ++j) { VALU(x0); VALU(x1); VALU(x2); VALU(x3); VALU(x4); VALU(x5); }
     }
+  } else if (role == 6) {
+    for (int it = 0; it < iters; ++it) { MFMA(acc0); MFMA(acc0); MFMA(acc0); MFMA(acc0); MFMA(acc0); MFMA(acc0); MFMA(acc0); MFMA(acc0); }
+  } else if (role == 7) {
+    for (int it = 0; it < iters; ++it) { MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1); MFMA(acc0); MFMA(acc1); }
   } else if (role == 5) {
     for (int it = 0; it < iters; ++it) {
 #define STEP3(acc) MFMA(acc); VALU(x0); VALU(x1); VALU(x2);
@@ -139,6 +144,9 @@ int main() {
   run_rate<3>("v_exp_f32, one dependent chain");
   printf("per iteration and wave: MFMA stream = 8 MFMAs 32x32x16 bf16 (256 matrix-pipe cycles), vector stream = 48 v_fmac_f32\n");
   run_coexec<1, 0>("one wave per SIMD: MFMAs only");
+  run_coexec<6, 0>("one wave per SIMD: MFMAs only, one dependent chain");
+  run_coexec<7, 0>("one wave per SIMD: MFMAs only, two alternating chains");
+  run_coexec<6, 6>("two waves per SIMD: both one dependent chain");
   run_coexec<2, 0>("one wave per SIMD: vector only");
   run_coexec<3, 0>("one wave per SIMD: interleaved 1 MFMA + 6 vector");
   run_coexec<4, 0>("one wave per SIMD: bursts 8 MFMAs then 48 vector");
