@@ -22,7 +22,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
   } while (0)
 
 // ---- part 1 ------------------------------------------------------------------------------------
-// MODE 0: 64 independent v_add_f32; 1: 64 v_add_f32 in one dependent chain; 2: 64 independent v_exp_f32; 3: dependent v_exp_f32
+// MODE 0: 64 independent v_add_f32; 1: 64 v_add_f32 in one dependent chain; 2: 64 independent v_exp_f32; 3: dependent v_exp_f32;
+// 4: 32 v_exp_f32 and 32 v_add_f32 alternating, all independent (does the transcendental unit run beside the ordinary one?)
 template <int MODE>
 __global__ void __launch_bounds__(256) valu_rate(int iters, float* out, float seed, long long* clk) {
   float x[16];
@@ -30,7 +31,16 @@ __global__ void __launch_bounds__(256) valu_rate(int iters, float* out, float se
   for (int i = 0; i < 16; ++i) x[i] = seed + i + threadIdx.x;
   const long long t0 = clock64();
   for (int it = 0; it < iters; ++it) {
-    if (MODE == 0 || MODE == 2) {
+    if (MODE == 4) {
+      float* y = x + 8;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          asm volatile("v_exp_f32 %0, %0" : "+v"(x[i]));
+          asm volatile("v_add_f32 %0, %0, %1" : "+v"(y[i]) : "v"(seed));
+        }
+    } else if (MODE == 0 || MODE == 2) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
@@ -142,6 +152,7 @@ int main() {
   run_rate<1>("v_add_f32, one dependent chain");
   run_rate<2>("v_exp_f32, independent");
   run_rate<3>("v_exp_f32, one dependent chain");
+  run_rate<4>("v_exp_f32 and v_add_f32 alternating (per instruction)");
   printf("per iteration and wave: MFMA stream = 8 MFMAs 32x32x16 bf16 (256 matrix-pipe cycles), vector stream = 48 v_fmac_f32\n");
   run_coexec<1, 0>("one wave per SIMD: MFMAs only");
   run_coexec<6, 0>("one wave per SIMD: MFMAs only, one dependent chain");
