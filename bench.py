@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # this script, so the figure is carried here for the workload it was taken on, with the file it was copied from
 TRAFFIC_SOURCE = "profiles/hbm_traffic_config2_llama8b_128k.md"
 MEASURED_TRAFFIC_BYTES = {
-    "config2_llama8b_128k": {0: 3.85e9, 3: 4.52e9},  # dominant-kernel index -> bytes (stage 1 as bench.py times it: without pooling; stage 3)
+    "config2_llama8b_128k": {0: 3.84e9, 3: 4.51e9},  # dominant-kernel index -> bytes (stage 1 as bench.py times it: without pooling; stage 3)
 }
 
 WORKLOADS = {
