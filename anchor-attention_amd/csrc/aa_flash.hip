@@ -781,345 +781,6 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   }  // query blocks of the work-group
 }
 
-#ifndef AA_PINGPONG
-#define AA_PINGPONG 0
-#endif
-#ifndef AA_PP_NOLOADS
-#define AA_PP_NOLOADS 0
-#endif
-#ifndef AA_PP_TRACE
-#define AA_PP_TRACE 0
-#endif
-
-// ---- ping-pong variant of the consecutive-key modes ---------------------------------------------------------------
-// Work-group = 8 waves = 256 query rows: waves 0-3 (group 0) own rows 0-127, waves 4-7 (group 1) rows 128-255; wave w
-// and wave w + 4 run on the same SIMD.  Time is cut into phases that end in a work-group barrier.  In a "burst" phase a
-// wave issues nothing but MFMAs - the scores of tile i and the P.V product of tile i-1, 32 MFMAs back to back - and in
-// a "soft-max" phase nothing but the vector work of tile i.  The two groups are one phase apart: while group 0 bursts
-// group 1 runs its soft-max and the other way round, so on every SIMD one wave feeds the matrix pipe and the other the
-// vector ALU, by construction and not by chance.
-//   phase 2i   : group 0 burst(i)    | group 1 soft-max(i-1)      burst(i)    = S(i) = K(i) Q^T ; O += V(i-1)^T P(i-1)^T
-//   phase 2i+1 : group 0 soft-max(i) | group 1 burst(i)
-// K(i) is read in phases 2i and 2i+1, V(i-1) in the same two; both are double-buffered (K(i) in K buffer i&1, V(i) in V
-// buffer i&1) and the loads of K(i+1) and V(i) are issued by all eight waves at the start of phase 2i and waited for at
-// the end of phase 2i+1: two phases of lead.  Group 0's rows end 128 keys earlier: it sits out the last two tiles.
-template <int MODE, typename T, int D>
-__global__ void __launch_bounds__(512, 1) flash_pp_kernel(const FlashArgs p) {
-  typedef typename T::vec8 vec8;
-  typedef __attribute__((address_space(3))) vec8 lds_vec8;
-  struct PpSmem { struct { char k[2][kTileBytes]; char v[3][kTileBytes]; } t; };
-  __shared__ __attribute__((aligned(16))) PpSmem sm;
-  constexpr int BM = 256;
-  static_assert(MODE != kSparse, "consecutive keys only");
-  constexpr int kKS = D / 16, kDB = D / 32, kNS = 2 * kKS, kNV = 4 * kDB;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grp = wave >> 2, wq = wave & 3;
-  const int half = lane >> 5;
-  const int c32 = lane & 31;
-
-  const int group = p.n_q_heads / p.n_kv_heads;
-  const int n_qunit = p.n_ctx / BM;
-  const int S = p.big_block;
-  uint32_t vid = xcd_remap(blockIdx.x, p.batch * p.n_kv_heads, group * n_qunit, group);
-  const int g = vid % group;  vid /= group;
-  int qunit = vid % n_qunit;  vid /= n_qunit;
-  const int kvh = vid % p.n_kv_heads;
-  const int b = vid / p.n_kv_heads;
-  qunit = n_qunit - 1 - qunit;  // longest rows first
-  const int hq = kvh * group + g;
-  const int R0 = qunit * BM;
-  const int bb = R0 / S;
-  const int64_t bh = (int64_t)b * p.n_q_heads + hq;
-  const int wr0 = R0 + grp * 128 + wq * 32;
-  const int my_row = wr0 + c32;
-
-  const uint16_t* qp = p.q + b * p.q_sb + hq * p.q_sh;
-  const char* kbase = reinterpret_cast<const char*>(p.k + b * p.k_sb + kvh * p.k_sh);
-  const char* vbase = reinterpret_cast<const char*>(p.v + b * p.v_sb + kvh * p.v_sh);
-  const uint32_t k_row_bytes = (uint32_t)p.k_sn * 2u, v_row_bytes = (uint32_t)p.v_sn * 2u;
-
-  // tiles of the work-group and of this wave's group
-  int n_init, n_tiles;
-  if (MODE == kAnchor) {
-    n_init = min(S, R0 + BM) / kBN;
-    n_tiles = n_init + (bb >= 1 ? (R0 + BM - bb * S) / kBN : 0);
-  } else {
-    n_init = 0;
-    n_tiles = (R0 + BM) / kBN;
-  }
-  const int n_mine = n_tiles - (grp == 0 ? 2 : 0);
-#define PP_TILE_KEY0(i) ((MODE == kAnchor) ? ((i) < n_init ? (i) * kBN : bb * S + ((i) - n_init) * kBN) : (i) * kBN)
-
-  // ---- tile loads ----------------------------------------------------------------------------------------------
-  // Only a bursting wave issues loads, one every eight MFMAs (issued all at once by all waves they queue up in the
-  // memory pipeline, about 40 cycles apiece, and every wave stalls for the length of the queue): group 0 brings the K
-  // tiles, group 1 the V tiles; wave wq of the group brings rows 16 wq .. 16 wq + 15 with four loads.
-  uint32_t t_voff[4];
-  const uint32_t t_row_bytes = grp == 0 ? k_row_bytes : v_row_bytes;
-#pragma unroll
-  for (int jj = 0; jj < 4; ++jj) {
-    const int row = 4 * jj + (lane >> 4);  // low four bits of the tile row
-    const uint32_t chunk = grp == 0 ? (uint32_t)((lane & 15) ^ (row & 15)) : (uint32_t)((lane & 15) ^ ((row & 7) << 1));
-    t_voff[jj] = (uint32_t)(lane >> 4) * t_row_bytes + (chunk & (uint32_t)(D / 8 - 1)) * 16u;
-  }
-  const char* t_base = grp == 0 ? kbase : vbase;
-  const uint32_t lds_tw = (grp == 0 ? lds_addr(sm.t.k[0]) : lds_addr(sm.t.v[0])) + 16 * wq * kRowBytes;
-  // load jj of this wave's share of tile i into buffer `slot` of its operand (K for group 0, V for group 1)
-  auto load_part = [&](const int i, const int slot, const int jj) {
-    const char* src = t_base + (uint64_t)(uint32_t)(PP_TILE_KEY0(i) + 16 * wq + 4 * jj) * t_row_bytes;
-    load16_to_lds(src, t_voff[jj], lds_tw + slot * kTileBytes + 4 * jj * kRowBytes);
-  };
-#pragma unroll
-  for (int jj = 0; jj < 4; ++jj) load_part(0, 0, jj);  // K(0) and V(0)
-
-  // ---- queries: B operand, pre-scaled into the exp2 domain ---------------------------------------------------------
-  vec8 qreg[kKS];
-  {
-    const bool chain = (MODE == kAnchor) && (p.scale_mode == 0);
-    const uint16_t* qrow = qp + (int64_t)my_row * p.q_sn + 8 * half;
-#pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) qreg[ks] = scale_q8<T>(*reinterpret_cast<const u32x4*>(qrow + 16 * ks), p.sm_scale, chain);
-  }
-  float m_run = -INFINITY, l_run = 0.f, m_ref = 0.f;
-  floatx16 acc[kDB], negm;
-#pragma unroll
-  for (int db = 0; db < kDB; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) negm[r] = 0.f;
-
-  // LDS read addresses: K of tile i in K buffer i & 1, V of tile i-1 in slot (i-1) % 3 of the V ring
-  uint32_t k_rd[kKS], v_rd[kDB];
-#pragma unroll
-  for (int ks = 0; ks < kKS; ++ks) k_rd[ks] = lds_addr(sm.t.k[0]) + c32 * kRowBytes + (((2 * ks + half) ^ (c32 & 15)) << 4);
-  {
-    const int r0 = 4 * half + ((lane & 15) >> 2);
-    const int y0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-#pragma unroll
-    for (int m = 0; m < kDB; ++m) v_rd[m] = lds_addr(sm.t.v[0]) + r0 * kRowBytes + (((4 * m + y0) ^ (r0 << 1)) << 4) + 8 * (lane & 1);
-  }
-  int32_t k_step = kTileBytes;
-  int v_slot = 2;  // ring slot of V(i-1) for the coming iteration i (i = 0 reads nothing); V(i+1) goes to slot (v_slot + 2) % 3
-
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();  // K(0) is in place
-
-#if AA_PP_TRACE
-  long long* trace = reinterpret_cast<long long*>(p.L_out + (int64_t)p.batch * p.n_q_heads * p.n_ctx) + wave * 128;
-  const bool traced = blockIdx.x == AA_PP_TRACE;
-#define PP_STAMP(k) if (traced && i >= 8 && i < 16 && lane == 0) { trace[(i - 8) * 16 + (k)] = clock64(); }
-#else
-#define PP_STAMP(k)
-#endif
-  // A phase ends in a bare barrier: every LDS read of the phase has been consumed by an MFMA already, and a wait on the
-  // LDS counter would also wait for the wave's own global -> LDS loads, which are meant to stay in flight.
-  auto phase_barrier = [&]() { asm volatile("s_barrier" ::: "memory"); };
-  floatx16 s0, s1;        // scores of the tile in flight between a burst and its soft-max
-  u32x4 pw0[2], pw1[2];   // P^T of the tile in flight between a soft-max and the next burst
-#define PP_FENCE __builtin_amdgcn_sched_barrier(0)
-
-  auto burst = [&](const int i) __attribute__((always_inline)) {
-    // this burst's loads: group 0 K(i+1) -> K buffer (i+1) & 1, group 1 V(i+1) -> ring slot (v_slot + 2) % 3
-    const bool do_load = !AA_PP_NOLOADS && i + 1 < n_tiles;
-    const int ld_slot = grp == 0 ? ((i + 1) & 1) : (v_slot == 0 ? 2 : v_slot - 1);
-    uint32_t v_cur[kDB];
-#pragma unroll
-    for (int m = 0; m < kDB; ++m) v_cur[m] = v_rd[m] + (uint32_t)v_slot * kTileBytes;
-    if (i < n_mine) {
-      vec8 ka[kNS];
-#define PP_K_FETCH(t) ka[t] = *(const lds_vec8*)(uintptr_t)(k_rd[(t) % kKS] + (uint32_t)(32 * ((t) / kKS) * kRowBytes))
-#pragma unroll
-      for (int n = 0; n < kDist; ++n) { const int t0 = (n & 1) * kKS + (n >> 1); PP_K_FETCH(t0); }
-      PP_FENCE;
-#pragma unroll
-      for (int n = 0; n < kNS; ++n) {  // the two chains alternate: s0, s1, s0, ...
-        const int t = (n & 1) * kKS + (n >> 1);
-        if (n + kDist < kNS) { const int t2 = ((n + kDist) & 1) * kKS + ((n + kDist) >> 1); PP_K_FETCH(t2); }
-        if (n & 1) s1 = T::mfma(ka[t], qreg[t % kKS], (t % kKS) == 0 ? negm : s1);
-        else s0 = T::mfma(ka[t], qreg[t % kKS], (t % kKS) == 0 ? negm : s0);
-        PP_FENCE;
-      }
-#undef PP_K_FETCH
-    }
-    PP_STAMP(12)
-    if (i >= 1 && i <= n_mine) {
-      shortx4 vlo[kNV], vhi[kNV];
-#define PP_V_SRC(x) (v_cur[(x) % kDB] + (uint32_t)((32 * ((x) / (2 * kDB)) + 16 * (((x) / kDB) & 1)) * kRowBytes))
-#define PP_V_FETCH(x)                                                                                    \
-  {                                                                                                      \
-    vlo[x] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(PP_V_SRC(x)));                       \
-    vhi[x] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(uintptr_t)(PP_V_SRC(x) + 8u * kRowBytes));      \
-  }
-#define PP_PV_MFMA(x, pw)                                                                                \
-  {                                                                                                      \
-    typedef short shortx8 __attribute__((ext_vector_type(8)));                                           \
-    const shortx8 av = __builtin_shufflevector(vlo[x], vhi[x], 0, 1, 2, 3, 4, 5, 6, 7);                  \
-    acc[(x) % kDB] = T::mfma(*reinterpret_cast<const vec8*>(&av), *reinterpret_cast<const vec8*>(&pw[((x) / kDB) & 1]), acc[(x) % kDB]); \
-  }
-#pragma unroll
-      for (int n = 0; n < kDist; ++n) PP_V_FETCH(n)
-      PP_FENCE;
-#pragma unroll
-      for (int n = 0; n < kNV; ++n) {
-        if (n + kDist < kNV) PP_V_FETCH(n + kDist)
-        if (n < 2 * kDB) { PP_PV_MFMA(n, pw0) } else { PP_PV_MFMA(n, pw1) }
-        PP_FENCE;
-      }
-#undef PP_V_SRC
-#undef PP_V_FETCH
-#undef PP_PV_MFMA
-    }
-    // The loads come last: a wave's LDS reads queue up behind its own global -> LDS loads until their data has arrived
-    // (measured: every load placed between the operand reads of a burst held the MFMA stream up for a memory latency);
-    // after a burst the wave reads no LDS for a whole soft-max phase.
-    PP_STAMP(13)
-    if (do_load) {
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) load_part(i + 1, ld_slot, jj);
-    }
-    return do_load;
-  };
-
-  auto softmax = [&](const int i) __attribute__((always_inline)) {
-    if (i >= n_mine) return;
-    const int key0 = PP_TILE_KEY0(i);
-    // causal mask (only tiles that reach past the wave's first row need it)
-    if (key0 + 63 > wr0) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int kk = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (kk > my_row) s0[r] = -INFINITY;
-        if (kk + 32 > my_row) s1[r] = -INFINITY;
-      }
-    }
-    float a0 = fmaxf(fmaxf(s0[0], s0[1]), s0[2]), a1 = fmaxf(fmaxf(s0[3], s0[4]), s0[5]);
-    float a2 = fmaxf(fmaxf(s0[6], s0[7]), s0[8]), a3 = fmaxf(fmaxf(s0[9], s0[10]), s0[11]);
-    float a4 = fmaxf(fmaxf(s0[12], s0[13]), s0[14]), a5 = fmaxf(fmaxf(s0[15], s1[0]), s1[1]);
-    float a6 = fmaxf(fmaxf(s1[2], s1[3]), s1[4]), a7 = fmaxf(fmaxf(s1[5], s1[6]), s1[7]);
-    float a8 = fmaxf(fmaxf(s1[8], s1[9]), s1[10]), a9 = fmaxf(fmaxf(s1[11], s1[12]), s1[13]);
-    const float a10 = fmaxf(s1[14], s1[15]);
-    a0 = fmaxf(fmaxf(a0, a1), a2);
-    a3 = fmaxf(fmaxf(a3, a4), a5);
-    a6 = fmaxf(fmaxf(a6, a7), a8);
-    a9 = fmaxf(a9, a10);
-    const float mx = max_with_other_half(fmaxf(fmaxf(a0, a3), fmaxf(a6, a9)));
-    if (__any(m_ref + mx > m_run)) {
-      // slow path: some row's max grew.  Lanes whose max did not move get shift 0 and alpha 1 (exact).
-      const float m_new = fmaxf(m_run, m_ref + mx);
-      const float alpha = fast_exp2(m_run - m_new);
-      const float shift = m_new - m_ref;
-      m_run = m_new;
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s0[r] -= shift; s1[r] -= shift; }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) negm[r] = -m_new;
-#pragma unroll
-      for (int db = 0; db < kDB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
-    }
-    float sum0 = 0.f, sum1 = 0.f;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const float e0 = fast_exp2(s0[4 * c + 0]), e1 = fast_exp2(s0[4 * c + 1]), e2 = fast_exp2(s0[4 * c + 2]), e3 = fast_exp2(s0[4 * c + 3]);
-      sum0 += e0; sum0 += e1; sum0 += e2; sum0 += e3;
-      pw0[c >> 1][2 * (c & 1) + 0] = T::pack(e0, e1);
-      pw0[c >> 1][2 * (c & 1) + 1] = T::pack(e2, e3);
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const float e0 = fast_exp2(s1[4 * c + 0]), e1 = fast_exp2(s1[4 * c + 1]), e2 = fast_exp2(s1[4 * c + 2]), e3 = fast_exp2(s1[4 * c + 3]);
-      sum1 += e0; sum1 += e1; sum1 += e2; sum1 += e3;
-      pw1[c >> 1][2 * (c & 1) + 0] = T::pack(e0, e1);
-      pw1[c >> 1][2 * (c & 1) + 1] = T::pack(e2, e3);
-    }
-    l_run += sum0;
-    l_run += sum1;
-  };
-  auto flip = [&]() {
-#pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) k_rd[ks] += k_step;
-    k_step = -k_step;
-    v_slot = v_slot == 2 ? 0 : v_slot + 1;
-  };
-
-  // ---- the phases ---------------------------------------------------------------------------------------------------
-  if (grp == 1) phase_barrier();  // phase 0 of group 1: nothing to compute yet
-  for (int i = 0;; ++i) {
-    PP_STAMP(0)
-    const bool loaded = burst(i);
-    PP_STAMP(1)
-    // Group 1's V(i) - requested one burst ago, needed two phases from now - must have landed; the loads of this burst may
-    // stay in flight (memory returns in order).  Group 0's K loads are waited for after its soft-max.
-    if (grp == 1) {
-      if (loaded) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    PP_STAMP(2)
-    phase_barrier();
-    PP_STAMP(3)
-    if (i == n_tiles) break;
-    softmax(i);
-    flip();
-    PP_STAMP(4)
-    if (grp == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // K(i+1), requested in this group's burst(i), has landed
-    PP_STAMP(5)
-    phase_barrier();
-    PP_STAMP(6)
-  }
-  if (grp == 0) phase_barrier();  // phase 2 n_tiles + 1 of group 0
-#undef PP_FENCE
-#undef PP_TILE_KEY0
-
-  // ---- epilogue -------------------------------------------------------------------------------------------------------
-  const float l_tot = l_run + xor32(l_run);
-  if (MODE == kAnchor) {
-    if (half == 0) {
-      p.M_out[bh * p.n_ctx + my_row] = m_run;
-      p.L_out[bh * p.n_ctx + my_row] = l_tot;
-    }
-    float* af = p.acc_out + ((bh * (p.n_ctx / 32) + my_row / 32) * (4 * kDB)) * 256 + lane * 4;
-#pragma unroll
-    for (int db = 0; db < kDB; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        floatx4 t;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) t[c] = acc[db][rg * 4 + c];
-        __builtin_nontemporal_store(t, reinterpret_cast<floatx4*>(af + (db * 4 + rg) * 256));
-      }
-  } else {
-    // out = bf16(acc / l), staged per wave in the (now idle) tile space: 8 waves x 32 rows x 256 bytes = all four buffers
-    char* ob = sm.t.k[0] + wave * 32 * kRowBytes;
-    constexpr int kChunkMask = D / 8 - 1;
-    const float inv = 1.0f / l_tot;
-#pragma unroll
-    for (int db = 0; db < kDB; ++db)
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        u32x2 w;
-        w[0] = T::pack(acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv);
-        w[1] = T::pack(acc[db][rg * 4 + 2] * inv, acc[db][rg * 4 + 3] * inv);
-        *reinterpret_cast<u32x2*>(ob + c32 * kRowBytes + (((4 * db + rg) ^ (c32 & kChunkMask)) << 4) + 8 * half) = w;
-      }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    uint16_t* op = p.out + b * p.o_sb + hq * p.o_sh;
-    constexpr int kLanesPerRow = D / 8, kRowsPerStore = 64 / kLanesPerRow;
-#pragma unroll
-    for (int it = 0; it < 32 / kRowsPerStore; ++it) {
-      const int r = it * kRowsPerStore + lane / kLanesPerRow, c = lane % kLanesPerRow;
-      const u32x4 w = *reinterpret_cast<const u32x4*>(ob + r * kRowBytes + ((c ^ (r & kChunkMask)) << 4));
-      __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(op + (int64_t)(wr0 + r) * p.o_sn + 8 * c));
-    }
-  }
-}
-
 #ifndef AA_SPARSE_QBLOCKS
 #define AA_SPARSE_QBLOCKS 4  // 128-row query blocks a stage-3 work-group handles one after the other (when the big block allows)
 #endif
@@ -1131,18 +792,6 @@ static hipError_t launch(const FlashArgs& args, hipStream_t stream) {
   if (MODE == kSparse) {
     const int per_big_block = a.big_block / 128;  // even for every supported geometry
     a.q_blocks_per_wg = per_big_block % AA_SPARSE_QBLOCKS == 0 ? AA_SPARSE_QBLOCKS : (per_big_block % 2 == 0 ? 2 : 1);
-  }
-  if (AA_PINGPONG && MODE != kSparse && !(MODE == kAnchor && a.qbar_out != nullptr)) {
-    constexpr int PM = MODE == kSparse ? kDense : MODE;
-    const dim3 grid((uint32_t)a.batch * a.n_q_heads * (a.n_ctx / 256)), block(512);
-    if (a.head_dim == 128) {
-      if (a.dtype == 0) hipLaunchKernelGGL((flash_pp_kernel<PM, Bf16, 128>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((flash_pp_kernel<PM, F16, 128>), grid, block, 0, stream, a);
-    } else {
-      if (a.dtype == 0) hipLaunchKernelGGL((flash_pp_kernel<PM, Bf16, 64>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((flash_pp_kernel<PM, F16, 64>), grid, block, 0, stream, a);
-    }
-    return hipGetLastError();
   }
   const dim3 grid((uint32_t)a.batch * a.n_q_heads * (a.n_ctx / (128 * a.q_blocks_per_wg))), block(256);
   if (a.head_dim == 128) {
