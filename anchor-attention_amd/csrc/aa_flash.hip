@@ -118,16 +118,24 @@ __device__ __forceinline__ void load16_to_lds(const char* base, const uint32_t b
 // wave-uniform head bases, `k_col`/`v_col` the byte offset of this thread's (swizzled) chunk inside a row,
 // `lds_k`/`lds_v` the LDS address of row 4*w of the destination tile.  Gathered tiles take their row numbers from
 // the LDS window of the index list (a dependent global load per tile would put a full memory latency on the
-// critical path of every tile).
+// critical path of every tile); the caller reads a tile's four row numbers per lane (`gather_keys`, see tile_gather_keys)
+// before it issues the tile's first load: a wave's LDS reads are served in order with its global -> LDS loads, so a row
+// number read after a load would arrive only when that load's data has.
+// the row numbers lane `tid` needs for the gathered tile at list position key0 (positions past the count hold 0: row 0,
+// masked later)
+__device__ __forceinline__ void tile_gather_keys(uint32_t (&keys)[4], const int32_t* idx_win, const int key0, const int tid) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) keys[j] = (uint32_t)idx_win[(key0 + (tid >> 4) + 16 * j) & (kIdxWin - 1)];
+}
+
 template <int MODE>
 __device__ __forceinline__ void tile_fetch_one(const int n, const char* kb, const char* vb, const uint32_t k_row_bytes,
                                                const uint32_t v_row_bytes, const uint32_t k_col, const uint32_t v_col, const int key0,
-                                               const int tid, const int32_t* idx_win, const uint32_t lds_k, const uint32_t lds_v,
+                                               const uint32_t* gather_keys, const uint32_t lds_k, const uint32_t lds_v,
                                                const uint32_t k_voff, const uint32_t v_voff) {
   const int j = n >> 1;  // load n: K (even n) or V (odd n) rows 16*j + ...
   if (MODE == kSparse) {
-    const int row = (tid >> 4) + 16 * j;
-    const uint32_t key = (uint32_t)idx_win[(key0 + row) & (kIdxWin - 1)];  // positions past the count hold 0 (row 0, masked later)
+    const uint32_t key = gather_keys[j];  // this lane's row of the tile's j-th block of 16 rows
     if ((n & 1) == 0) load16_to_lds(kb, __umul24(key, k_row_bytes) + k_col, lds_k + 16 * j * kRowBytes);
     else load16_to_lds(vb, __umul24(key, v_row_bytes) + v_col, lds_v + 16 * j * kRowBytes);
   } else {
@@ -320,9 +328,11 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
   const uint32_t q_voff = (uint32_t)(tid >> 4) * q_row_bytes + (uint32_t)((tid & 15) & (D / 8 - 1)) * 16u;
   if (n_tiles > 0 && !chained) {
     const uint32_t first = MODE == kSparse ? (uint32_t)cur * kTileBytes : 0u;
+    uint32_t keys0[4] = {0u, 0u, 0u, 0u};
+    if (MODE == kSparse) tile_gather_keys(keys0, sm.idx, 0, tid);
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), tid, sm.idx, lds_k0 + first,
+      tile_fetch_one<MODE>(j, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, AA_TILE_KEY0(0), keys0, lds_k0 + first,
                            lds_v0 + first, k_voff, v_voff);
   }
   // the accumulator state: the youngest loads in flight, first needed by the first P.V product
@@ -479,6 +489,8 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     // (selects, not branches: the eight slots stay straight-line code; the base address is scalar, and the vector offset
     // is chosen once per tile and operand kind)
     const uint32_t k_voff_sel = fetch_queries ? q_voff : k_voff, v_voff_sel = fetch_queries ? q_voff : v_voff;
+    uint32_t keys_next[4] = {0u, 0u, 0u, 0u};  // (sparse) row numbers of the next tile, read before the tile's first load is issued
+    if (MODE == kSparse) tile_gather_keys(keys_next, sm.idx, key0_next, tid);
 #define AA_FETCH_ONE(n)                                                                                               \
   if (MODE == kAnchor) {                                                                                              \
     const int j_ = (n) >> 1;                                                                                          \
@@ -488,7 +500,7 @@ __global__ void __launch_bounds__(256, 2) flash_kernel(const FlashArgs p) {
     load16_to_lds(fetch_queries ? q_ : kv_, ((n) & 1) ? v_voff_sel : k_voff_sel,                                      \
                   (((n) & 1) ? lds_v0 : lds_k0) + (buf ^ 1) * kTileBytes + 16 * j_ * kRowBytes);                      \
   } else {                                                                                                            \
-    tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, tid, sm.idx,             \
+    tile_fetch_one<MODE>(n, kbase, vbase, k_row_bytes, v_row_bytes, k_col, v_col, key0_next, keys_next,               \
                          lds_k0 + (buf ^ 1) * kTileBytes, lds_v0 + (buf ^ 1) * kTileBytes, k_voff, v_voff);           \
   }
     // (a wave whose rows all lie above this tile - two of the four waves on the last tile of a causal work-group -
