@@ -7,6 +7,8 @@ operator's kernels can be read against a practical ceiling as well as against th
   * bf16 GEMMs (hipBLASLt through torch.matmul) on N(0,1) operands and on all-zero operands - the difference
     is the power a matrix pipe draws when its inputs toggle;
   * the framework's dense causal attention and this library's own dense kernel on the same shape;
+  * this library's own dense kernel on N(0,1), on all-zero and on half-zero operands: the same instruction stream at
+    the clocks the power management grants for each kind of data;
   * streaming element-wise kernels at several read:write mixes (the HBM rates a memory-bound kernel can expect).
 
     python bench_reference_points.py            # prints one JSON object
@@ -70,7 +72,18 @@ def main():
 
     ms = _time_ms(own, 5, warm=2)
     out["own_dense_causal_32k"] = {"ms": ms, "tflops": flops / ms / 1e9}
-    del q, k, v, o
+    # the same kernel, the same number of instructions, other operand data
+    by_data = {}
+    zq, zk, zv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    for name, (q_, k_, v_) in (("all-zero operands", (zq, zk, zv)), ("N(0,1) q and k, zero v", (q, k, zv)),
+                               ("zero q and k, N(0,1) v", (zq, zk, v)), ("N(0,1) operands", (q, k, v))):
+        def own_on():
+            _hip.check(lib.aa_dense_causal_fwd(*_hip.t3(q_), *_hip.t3(k_), *_hip.t3(v_), *_hip.t3(o), 1, hq, hkv, n_ctx, d,
+                                               d ** -0.5, _hip.AA_DTYPE_BF16, stream))
+        ms = _time_ms(own_on, 5, warm=2)
+        by_data[name] = {"ms": ms, "tflops": flops / ms / 1e9}
+    out["own_dense_causal_32k_by_operand_data"] = by_data
+    del q, k, v, o, zq, zk, zv
 
     # streaming kernels on 1 GiB fp32 tensors
     n = 2 ** 28
