@@ -192,6 +192,47 @@ def staged_pass(q, k, v, theta, steps, out):
     return st_ms, int(counts.sum())
 
 
+def stage1_on_zero_operands(dev, name, dtype):
+    """Stage 1 of the workload's shape on all-zero q, k, v: the same instruction stream (the kernel's control flow does not
+    depend on the data), but operands that do not toggle, so the power management lets the chip hold its nominal clock.
+    What this leg reports is therefore the kernel's efficiency per cycle; the headline figures are what the same kernel
+    gets at the clock the chip grants for real data.  The vendor GEMM is timed on all-zero operands next to it."""
+    import torch
+    from anchor_attn.src.ops import anchor_step_1_2_v2 as st
+    n_ctx, hq, hkv = WORKLOADS[name][0], WORKLOADS[name][1], WORKLOADS[name][2]
+    D = workload_head_dim(name)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    q = torch.zeros((1, hq, n_ctx, D), dtype=tdt, device=dev)
+    k = torch.zeros((1, hkv, n_ctx, D), dtype=tdt, device=dev)
+    v = torch.zeros((1, hkv, n_ctx, D), dtype=tdt, device=dev)
+    sm = 1.0 / math.sqrt(D)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    for i in range(8):
+        if i == 3:
+            ev[0].record()
+        L, M, Acc = st.anchor_attn_step_1(q, k, v, 1, 1, 128, 16, 1, hq, n_ctx, D, sm)
+        del L, M, Acc
+    ev[1].record()
+    torch.cuda.synchronize()
+    ms = ev[0].elapsed_time(ev[1]) / 5
+    f1 = flops(hq, n_ctx, 0, D=D)[0]
+    del q, k, v
+    n = 16384
+    a = torch.zeros((n, n), dtype=torch.bfloat16, device=dev)
+    b = torch.zeros((n, n), dtype=torch.bfloat16, device=dev)
+    c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
+    for i in range(8):
+        if i == 3:
+            ev[0].record()
+        torch.matmul(a, b, out=c)
+    ev[1].record()
+    torch.cuda.synchronize()
+    gemm_tflops = 2.0 * n ** 3 / (ev[0].elapsed_time(ev[1]) / 5) / 1e9
+    tflops = f1 / ms / 1e9
+    return {"ms": ms, "tflops": tflops, "frac_of_mfma_peak": tflops / PEAK_BF16_TFLOPS,
+            "gemm_16384_on_zero_operands_tflops": gemm_tflops, "frac_of_that_gemm": tflops / gemm_tflops}
+
+
 def stage3_dense_regime(dev, seed, dtype):
     """Stage 3 where it is bound by the matrix pipe: the 32k-token Llama shape with the literal reading of the generator
     (no shared query component), under which nearly every candidate key passes the difference test (ratio ~0.92), so the
@@ -231,6 +272,9 @@ def main():
     ap.add_argument("--no-dense-regime", action="store_true",
                     help="skip the extra leg that times stage 3 where it is bound by the matrix pipe (32k tokens, "
                          "nearly every key selected)")
+    ap.add_argument("--no-zero-operands", action="store_true",
+                    help="skip the extra leg that times stage 1 (and the vendor GEMM) on all-zero operands, i.e. at the "
+                         "nominal clock: the kernel's efficiency per cycle")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 1 GiB device copies (a kernel of known traffic) so that rocprofv3 "
                          "FETCH_SIZE/WRITE_SIZE readings of the attention kernels can be scaled")
@@ -323,6 +367,8 @@ def main():
     if not args.no_dense_regime:
         del q, k, v, out
         rec["stage3_dense_regime"] = stage3_dense_regime(dev, args.seed, args.dtype)
+    if not args.no_zero_operands:
+        rec["stage1_on_zero_operands"] = stage1_on_zero_operands(dev, args.workload, args.dtype)
     if not args.no_gemm_ref:
         rec["mfma_reference"] = gemm_reference(dev)
         roof["frac_of_gemm_reference"] = roof["achieved"] / rec["mfma_reference"]["tflops"]
